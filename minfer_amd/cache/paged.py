@@ -55,10 +55,16 @@ class KVRequest:
     head_dim: int
     window: Optional[int] = None      # None: all earlier positions
     v_head_dim: Optional[int] = None  # width of a value row where it is not that of a key row
+    chunk: Optional[int] = None       # a position reads only its own chunk of this many positions, counted from 0
 
     @property
     def value_dim(self) -> int:
         return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    @property
+    def gives_pages_back(self) -> bool:
+        """Whether positions fall out of every later query's sight as a sequence grows."""
+        return self.window is not None or self.chunk is not None
 
 
 @dataclass(frozen=True)
@@ -140,10 +146,13 @@ class KVGroup:
 
     def first_needed_page(self, length: int) -> int:
         """Lowest logical page a query at position >= length can still read."""
-        w = self.request.window
-        if w is None:
-            return 0
-        return max(0, length - w + 1) // PAGE
+        w, c = self.request.window, self.request.chunk
+        first = 0
+        if w is not None:
+            first = max(0, length - w + 1)
+        if c is not None:
+            first = max(first, length // c * c)       # later positions lie in this chunk or behind it
+        return first // PAGE
 
     def pages_missing(self, slot: int, new_len: int) -> int:
         return max(0, (new_len + PAGE - 1) // PAGE - len(self.pages[slot]))
@@ -253,7 +262,7 @@ class Cache:
         for slot, n in new_lengths.items():
             self.lengths[slot] = n
             for g in self.groups:
-                if g.request.window is not None:
+                if g.request.gives_pages_back:
                     g.drop_left_of_window(slot, n)
 
     def truncate(self, slot: int, length: int) -> None:

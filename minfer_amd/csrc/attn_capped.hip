@@ -9,6 +9,8 @@
 //   v <- (1 - lambda) v + lambda v_first, where a layer blends;
 //   s_j = cap tanh((q . k_j) scale temp[h] / cap), keys j with 0 <= p - j < window, ordinary softmax,
 //   o = sum_j p_j v_j.
+// The attention kernels also take a mask in chunks (a token sees the keys of its own chunk of `chunk`
+// positions counted from 0, up to itself) and a penalty on distance, s_j -= a[h] ln(1 + b[h] (p - j)).
 //
 // `qkv_conv_prep_kernel`: one workgroup per (token, head of q, k or v); convolution of the head's channels
 // into LDS, then rotation, blending, the cache write and q rounded to the run type.
@@ -122,7 +124,8 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
     const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ page_table,
     int pt_stride, const int* __restrict__ positions, const int* __restrict__ seq_of_tok,
     const float* __restrict__ temp, T* __restrict__ out, float* __restrict__ part, int nh, int nk, int D, int V,
-    int VP, float scale, float cap, int window, int n_splits, int split_len) {
+    int VP, float scale, float cap, int window, int chunk, const float* __restrict__ far_a,
+    const float* __restrict__ far_b, int n_splits, int split_len) {
   extern __shared__ float lds[];
   float* sq = lds;                              // [GC][D]
   float* sc = sq + MF_CAP_GC * D;               // [GC][KEYS]
@@ -141,7 +144,8 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
 
   const int p = positions[t];
   const int* pt = page_table + (size_t)seq_of_tok[t] * pt_stride;
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  int lo = window > 0 ? max(0, p - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, p / chunk * chunk);
   // a windowed token's splits start at its window's first key, so that all of them have keys
   const int j_begin = lo + split * split_len;
   const int j_end = min(p + 1, j_begin + split_len);
@@ -156,6 +160,12 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
   float tm[MF_CAP_GC];
 #pragma unroll
   for (int g = 0; g < MF_CAP_GC; ++g) tm[g] = g < gcount ? scale * temp[h0 + g] : 0.f;
+  float fa[MF_CAP_GC], fb[MF_CAP_GC];      // the penalty on distance, per head
+#pragma unroll
+  for (int g = 0; g < MF_CAP_GC; ++g) {
+    fa[g] = (far_a && g < gcount) ? far_a[h0 + g] : 0.f;
+    fb[g] = (far_a && g < gcount) ? far_b[h0 + g] : 0.f;
+  }
   const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
   __syncthreads();
 
@@ -194,6 +204,7 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
       for (int g = 0; g < MF_CAP_GC; ++g) {
         float x = s[g] * tm[g];
         if (cap > 0.f) x = cap * tanhf(x * inv_cap);
+        if (far_a && valid) x -= fa[g] * log1pf(fb[g] * (float)(p - j));
         sc[g * MF_CAP_KEYS + threadIdx.x] = valid ? x : -INFINITY;
       }
     }
@@ -334,10 +345,11 @@ MF_API int mf_qkv_conv_prep(const float* qkv, const float* conv_w, int taps, flo
 MF_API int mf_capped_attn(const void* q, const void* kc, const void* vc, const int* page_table, int pt_stride,
                           const int* positions, const int* seq_of_tok, const float* temp, void* out, float* part,
                           int is_bf16, int n_tok, int nh, int nk, int D, int V, float scale, float cap, int window,
-                          int n_splits, int split_len, hipStream_t stream) {
+                          int chunk, const float* far_a, const float* far_b, int n_splits, int split_len,
+                          hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (nk <= 0 || nh % nk || D <= 0 || D > 512 || V <= 0 || V > 256 || n_splits < 1 || n_splits > 64 ||
-      split_len < 1 || (n_splits > 1 && !part) || !temp)
+      split_len < 1 || (n_splits > 1 && !part) || !temp || chunk < 0 || (far_a != nullptr) != (far_b != nullptr))
     return (int)hipErrorInvalidValue;
   int VP = 1;
   while (VP < V) VP *= 2;
@@ -348,7 +360,8 @@ MF_API int mf_capped_attn(const void* q, const void* kc, const void* vc, const i
   if (is_bf16) {
     capped_attn_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table,
                                                          pt_stride, positions, seq_of_tok, temp, (bf16*)out, part, nh, nk,
-                                                         D, V, VP, scale, cap, window, n_splits, split_len);
+                                                         D, V, VP, scale, cap, window, chunk, far_a, far_b, n_splits,
+                                                         split_len);
     rc = mf_launch_status();
     if (rc == 0 && n_splits > 1) {
       attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64 * ((V + 63) / 64), 0, stream>>>(part, (bf16*)out, V, n_splits);
@@ -357,7 +370,8 @@ MF_API int mf_capped_attn(const void* q, const void* kc, const void* vc, const i
   } else {
     capped_attn_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)kc, (const float*)vc, page_table,
                                                           pt_stride, positions, seq_of_tok, temp, (float*)out, part, nh,
-                                                          nk, D, V, VP, scale, cap, window, n_splits, split_len);
+                                                          nk, D, V, VP, scale, cap, window, chunk, far_a, far_b, n_splits,
+                                                         split_len);
     rc = mf_launch_status();
     if (rc == 0 && n_splits > 1) {
       attn_tokens::attn_combine_kernel<float><<<n_tok * nh, 64 * ((V + 63) / 64), 0, stream>>>(part, (float*)out, V, n_splits);

@@ -1,7 +1,9 @@
 // Windowed, capped attention for many query tokens per sequence (prompts and their portions), bfloat16, on
 // the gfx950 matrix cores, for keys of MF_CAPM_D and values of MF_CAPM_V values (multiples of 16, given at
 // compile time: the library is built for a model's sizes).  Semantics as `capped_attn_kernel`:
-// s = cap tanh(q . k scale temp[h] / cap), keys j with 0 <= p - j < window, softmax, o = sum p_j v_j.
+// s = cap tanh(q . k scale temp[h] / cap), keys j with 0 <= p - j < window, softmax, o = sum p_j v_j; with
+// `chunk`, a token sees the keys of its own chunk of that many positions only; with `far_a`, `far_b`,
+// s -= far_a[h] ln(1 + far_b[h] (p - j)).
 //
 // A wave (a workgroup of its own) owns 16 consecutive new tokens of one sequence times RB query heads of one kv
 // head and walks the tokens' keys 32 at a time (half a page), with no LDS and no barrier; the key rows of a
@@ -47,7 +49,8 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_seq, const int* __restrict__ tile_q0, int n_tiles,
     const float* __restrict__ temp, bf16* __restrict__ out, float* __restrict__ part, int n_splits, int split_len,
-    int nh, int nk, float scale, float cap, int window) {
+    int nh, int nk, float scale, float cap, int window, int chunk, const float* __restrict__ far_a,
+    const float* __restrict__ far_b) {
   const int lane = threadIdx.x & 63;
   const int tile = blockIdx.x;                    // a workgroup is one wave: the waves drift apart freely
   if (tile >= n_tiles) return;
@@ -67,7 +70,9 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
   const int p_mine = p0 + col;                    // this lane's token (rows beyond `rows` are masked out)
   const bool row_ok = col < rows;
   const int* pt = page_table + (size_t)b * pt_stride;
-  const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, p0 / chunk * chunk);          // the first token's chunk starts first
+  const int chunk_lo = chunk > 0 ? p_mine / chunk * chunk : 0;
   // with key splits (steps of few tokens), this wave takes the keys [k_first, k_stop) of the tile's, counted
   // in half pages from the one that holds the first key
   const int split = blockIdx.z;
@@ -88,6 +93,12 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
   float sc[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) sc[r] = scale * temp[h0 + r];
+  float fa[RB], fb[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    fa[r] = far_a ? far_a[h0 + r] : 0.f;
+    fb[r] = far_a ? far_b[h0 + r] : 0.f;
+  }
   const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
 
   floatx4 oacc[RB][NVT];
@@ -136,10 +147,12 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     }
     // which of this lane's 8 keys its token sees: slot j < 4: key kb + 4 g + j, else kb + 16 + 4 g + j - 4
     bool seen[8];
+    float dist[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int key = kb + (j < 4 ? 4 * g + j : 16 + 4 * g + j - 4);
-      seen[j] = row_ok && key <= p_mine && (window <= 0 || p_mine - key < window);
+      seen[j] = row_ok && key <= p_mine && (window <= 0 || p_mine - key < window) && key >= chunk_lo;
+      dist[j] = (float)max(0, p_mine - key);
     }
     bf16x8 pf[RB];
 #pragma unroll
@@ -156,6 +169,7 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
       for (int j = 0; j < 8; ++j) {
         float y = (j < 4 ? s0[j] : s1[j - 4]) * sc[r];
         if (cap > 0.f) y = cap * fast_tanh(y * inv_cap);
+        if (far_a) y -= fa[r] * __logf(1.0f + fb[r] * dist[j]);
         x[j] = seen[j] ? y : -INFINITY;
         mx = fmaxf(mx, x[j]);
       }
@@ -240,10 +254,12 @@ MF_API int mf_capped_mfma_sizes(int* d, int* v) {
 MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const int* page_table, int pt_stride,
                           const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0,
                           int n_tiles, const float* temp, void* out, float* part, int n_splits, int split_len, int n_tok,
-                          int nh, int nk, int d, int v, float scale, float cap, int window, hipStream_t stream) {
+                          int nh, int nk, int d, int v, float scale, float cap, int window, int chunk, const float* far_a,
+                          const float* far_b, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (d != D || v != V || nk <= 0 || nh % nk || !temp || n_splits < 1 || n_splits > 64 ||
-      (n_splits > 1 && (!part || split_len < 32 || split_len % 32)))
+      (n_splits > 1 && (!part || split_len < 32 || split_len % 32)) || chunk < 0 ||
+      (far_a != nullptr) != (far_b != nullptr))
     return (int)hipErrorInvalidValue;
   const int G = nh / nk;
   // heads of a kv head a wave takes together: four where that still leaves waves for all SIMDs
@@ -253,7 +269,7 @@ MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const i
 #define MF_GO(RB)                                                                                                          \
   capped_mfma_kernel<RB><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, \
                                                    cu_seqlens, start_pos, tile_seq, tile_q0, n_tiles, temp, (bf16*)out, part, \
-                                                   n_splits, split_len, nh, nk, scale, cap, window)
+                                                   n_splits, split_len, nh, nk, scale, cap, window, chunk, far_a, far_b)
   if (rb == 4) MF_GO(4);
   else if (rb == 2) MF_GO(2);
   else MF_GO(1);

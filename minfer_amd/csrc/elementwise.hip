@@ -688,3 +688,16 @@ MF_API int mf_weighted_sum(const void* const* ptrs, int n, int n_indexed, const 
   }
   return 0;
 }
+
+// ---------------------------------------------------------------- rows added into rows
+// h[r][:] += x[r][:], both 32-bit (an earlier state of the residual stream that joins it again)
+__global__ __launch_bounds__(256) void add_rows_kernel(float* __restrict__ h, const float* __restrict__ x, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) h[i] += x[i];
+}
+
+MF_API int mf_add_rows(float* h, const float* x, size_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  add_rows_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(h, x, n);
+  return mf_launch_status();
+}

@@ -5,7 +5,11 @@
 // groups can be chosen; the `top` best of those are chosen (ties go to the lower index) and weighted
 // by their scores over the sum of the chosen scores (+ 1e-20).  One wave per token.
 //
-// Expert: g = min(gate, limit), u = clamp(up, -limit, limit), y = g sigmoid(1.702 g) (u + 1).
+// A router may add a bias per expert to its logits.  With one group, all of it kept, the weights are the
+// softmax over the chosen logits alone (the scores' common divisor cancels).
+//
+// Expert: g = min(gate, limit), u = clamp(up, -limit, limit), y = g sigmoid(1.702 g) (u + 1); or, with
+// `act` 1, the plain gated form y = silu(gate) up.
 // `moe_act_kernel` applies it to the gate|up sums of every expert and multiplies by the token's
 // weight for that expert (0 where it was not chosen), so that one product with the experts' down
 // matrices side by side gives the weighted sum of the chosen experts' outputs.
@@ -46,7 +50,8 @@ __device__ __forceinline__ void load4(const float* __restrict__ p, float (&d)[4]
 // x [tokens][K] in the run type, router [E][K] float32: a workgroup per token; its four waves form the E
 // logits (a wave an expert at a time, lanes over K in runs of 4, sums in 32-bit), then the first wave decides.
 template <typename XT>
-__global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x, const float* __restrict__ router, int K,
+__global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x, const float* __restrict__ router,
+                                                       const float* __restrict__ bias, int K,
                                                        float* __restrict__ dense, int* __restrict__ chosen,
                                                        float* __restrict__ weights, int E, int n_groups, int keep,
                                                        int top) {
@@ -69,7 +74,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x
       for (int i = lane; i < K; i += 64) a = fmaf(wr[i], to_f32(xr[i]), a);
     }
     a = wave_sum(a);
-    if (lane == 0) s[e] = a;
+    if (lane == 0) s[e] = bias ? a + bias[e] : a;
   }
   __syncthreads();
   if (wv != 0) return;              // from here on one wave: MF_WAVE_SYNC where the block form has a barrier
@@ -126,7 +131,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x
   }
 }
 
-__device__ __forceinline__ float expert_act(float g, float u, float limit) {
+#define MF_MOE_ACT_CLAMPED 0
+#define MF_MOE_ACT_SILU 1
+
+__device__ __forceinline__ float expert_act(float g, float u, float limit, int act) {
+  if (act == MF_MOE_ACT_SILU) return g * (1.0f / (1.0f + expf(-g))) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
@@ -135,14 +144,14 @@ __device__ __forceinline__ float expert_act(float g, float u, float limit) {
 // gu [tokens][E][2 F] (an expert's gate sums, then its up sums); dense [tokens][E]; y [tokens][E F]
 template <typename OT>
 __global__ __launch_bounds__(256) void moe_act_kernel(const float* __restrict__ gu, const float* __restrict__ dense,
-                                                      OT* __restrict__ y, int E, int F, float limit) {
+                                                      OT* __restrict__ y, int E, int F, float limit, int act) {
   const int t = blockIdx.x;
   const float* row = gu + (size_t)t * E * 2 * F;
   for (int i = blockIdx.y * 256 + threadIdx.x; i < E * F; i += gridDim.y * 256) {
     const int e = i / F, f = i % F;
     const float wgt = dense[(size_t)t * E + e];
     float v = 0.f;
-    if (wgt != 0.f) v = wgt * expert_act(row[(size_t)e * 2 * F + f], row[(size_t)e * 2 * F + F + f], limit);
+    if (wgt != 0.f) v = wgt * expert_act(row[(size_t)e * 2 * F + f], row[(size_t)e * 2 * F + F + f], limit, act);
     y[(size_t)t * E * F + i] = from_f32<OT>(v);
   }
 }
@@ -188,7 +197,7 @@ __device__ __forceinline__ int next_pair(unsigned long long& m0, unsigned long l
 template <typename WT>
 __global__ __launch_bounds__(256) void moe_sparse_up_kernel(const WT* __restrict__ x, const WT* __restrict__ gate_up,
                                                             const int* __restrict__ chosen, WT* __restrict__ y,
-                                                            int n_pairs, int top, int F, int K, float limit) {
+                                                            int n_pairs, int top, int F, int K, float limit, int act) {
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int f = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(256) void moe_sparse_up_kernel(const WT* __restrict
     if (m0 | m1) {
       const int pr = next_pair(m0, m1);
       const float g = wave_sum(ag[j]), u = wave_sum(au[j]);
-      if (lane == 0) y[(size_t)pr * F + f] = from_f32<WT>(expert_act(g, u, limit));
+      if (lane == 0) y[(size_t)pr * F + f] = from_f32<WT>(expert_act(g, u, limit, act));
     }
   }
 }
@@ -327,48 +336,50 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 }
 
 // ------------------------------------------------------------------ entry points
-MF_API int mf_moe_route(const void* x, int x_is_bf16, const float* router, int K, float* dense, int* chosen,
+MF_API int mf_moe_route(const void* x, int x_is_bf16, const float* router, const float* bias, int K, float* dense, int* chosen,
                         float* weights, int n_tok, int E, int n_groups, int keep, int top, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (K <= 0 || E <= 0 || E > MF_MOE_MAX_EXPERTS || n_groups <= 0 || E % n_groups || keep <= 0 || keep > n_groups || top <= 0 ||
       top > 64 || top > keep * (E / n_groups))
     return (int)hipErrorInvalidValue;
   if (x_is_bf16)
-    moe_route_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)x, router, K, dense, chosen, weights, E, n_groups, keep, top);
+    moe_route_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)x, router, bias, K, dense, chosen, weights, E, n_groups, keep, top);
   else
-    moe_route_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)x, router, K, dense, chosen, weights, E, n_groups, keep, top);
+    moe_route_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)x, router, bias, K, dense, chosen, weights, E, n_groups, keep, top);
   return mf_launch_status();
 }
 
 MF_API int mf_moe_act(const float* gu, const float* dense, void* y, int y_is_bf16, int n_tok, int E, int F, float limit,
-                      hipStream_t stream) {
+                      int act, hipStream_t stream) {
   if (n_tok <= 0 || E <= 0 || F <= 0) return 0;
+  if (act != MF_MOE_ACT_CLAMPED && act != MF_MOE_ACT_SILU) return (int)hipErrorInvalidValue;
   int by = (E * F + 255) / 256;
   if (by > 64) by = 64;
   dim3 grid(n_tok, by);
   if (y_is_bf16)
-    moe_act_kernel<bf16><<<grid, 256, 0, stream>>>(gu, dense, (bf16*)y, E, F, limit);
+    moe_act_kernel<bf16><<<grid, 256, 0, stream>>>(gu, dense, (bf16*)y, E, F, limit, act);
   else
-    moe_act_kernel<float><<<grid, 256, 0, stream>>>(gu, dense, (float*)y, E, F, limit);
+    moe_act_kernel<float><<<grid, 256, 0, stream>>>(gu, dense, (float*)y, E, F, limit, act);
   return mf_launch_status();
 }
 
 MF_API int mf_moe_sparse(const void* x, const void* gate_up, const void* down, const int* chosen, const float* weights,
                          void* y, float* rows, float* out, int is_bf16, int n_tok, int top, int E, int F, int K, int N,
-                         float limit, hipStream_t stream) {
+                         float limit, int act, hipStream_t stream) {
   if (n_tok <= 0) return 0;
+  if (act != MF_MOE_ACT_CLAMPED && act != MF_MOE_ACT_SILU) return (int)hipErrorInvalidValue;
   if (top <= 0 || E <= 0 || F <= 0 || K <= 0 || N <= 0 || n_tok > MF_MOE_SPARSE_TOKENS || n_tok * top > MF_MOE_SPARSE_PAIRS ||
       !y || !rows)
     return (int)hipErrorInvalidValue;
   dim3 g1(E, (F + 3) / 4), g2(E, (N + 3) / 4);
   const int pairs = n_tok * top;
   if (is_bf16) {
-    moe_sparse_up_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, (const bf16*)gate_up, chosen, (bf16*)y, pairs, top, F, K, limit);
+    moe_sparse_up_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, (const bf16*)gate_up, chosen, (bf16*)y, pairs, top, F, K, limit, act);
     int rc = mf_launch_status();
     if (rc) return rc;
     moe_sparse_down_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)y, (const bf16*)down, chosen, rows, pairs, F, N);
   } else {
-    moe_sparse_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)y, pairs, top, F, K, limit);
+    moe_sparse_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)y, pairs, top, F, K, limit, act);
     int rc = mf_launch_status();
     if (rc) return rc;
     moe_sparse_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, chosen, rows, pairs, F, N);

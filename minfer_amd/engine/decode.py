@@ -159,12 +159,12 @@ class DecodeSession:
         # A page table row changes only when its sequence starts a new page (or, in a windowed
         # group, gives one back): that is the only time the host touches the tables.
         grows = [s for s, n in new_len.items() if (n - 1) % PAGE == 0]
-        windowed = any(g.request.window is not None for g in cache.groups)
+        windowed = any(g.request.gives_pages_back for g in cache.groups)
         if grows:
             cache.reserve({s: new_len[s] for s in grows})
         if grows or windowed or not self._host_tables:
             for g in cache.groups:
-                if self._host_tables and not grows and g.request.window is None:
+                if self._host_tables and not grows and not g.request.gives_pages_back:
                     continue
                 rows = cache.page_rows(g, self.slots, self.n_cols)
                 if self._host_tables.get(id(g)) != rows:

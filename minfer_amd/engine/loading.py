@@ -102,6 +102,8 @@ def random_model(config: Union[Dict[str, Any], Any], seed: int = 0, dtype="bfloa
             return torch.ones(ts.shape, dtype=dt, device=device)
         if ts.init == "zeros":
             return torch.zeros(ts.shape, dtype=dt, device=device)
+        if ts.init == "halves":
+            return torch.full(ts.shape, 0.5, dtype=dt, device=device)
         t = torch.empty(ts.shape, dtype=dt, device=device)
         ops.fill_normal(t, tensor_seed(seed, name), config.random_init_std(name), round_bf16=True)
         return t

@@ -132,13 +132,22 @@ class DecoderModel:
         s = self.spec
         h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.rt.device)
         self.embedding.forward(ctx.token_ids, h, ctx)
+        first = None
+        if any(e.adds_embedding for e in s.schedule):       # the embedding output joins the stream again later
+            first = torch.empty_like(h)
+            self.embedding.forward(ctx.token_ids, first, ctx)
         rows = ctx.logit_rows
         last = len(s.schedule) - 1
         ctx.norm_ahead = None
         for n, e in enumerate(s.schedule):
             keep = rows if (n == last and rows is not None) else None
             # the norm that reads the stream behind this block: the next block's first one, or the final one
-            ctx.norm_after_block = (self.final_norm if n == last else self.blocks[s.schedule[n + 1].block].first_norm())
+            ctx.norm_after_block = (self.final_norm if n == last else
+                                    None if s.schedule[n + 1].adds_embedding else
+                                    self.blocks[s.schedule[n + 1].block].first_norm())
+            if e.adds_embedding:
+                ops.add_rows(h, first)
+                ctx.norm_ahead = None
             h = self.blocks[e.block].forward(h, ctx, e.cache, e.writes_cache, keep_rows=keep)
             ahead = ctx.norm_ahead
             if ahead is not None and (ahead.norm is not ctx.norm_after_block or ahead.h is not h):

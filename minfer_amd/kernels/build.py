@@ -36,6 +36,8 @@ LIBRARIES: Dict[str, str] = {
     "linear_attention": "linear_attention.hip",
     "attn_capped": "attn_capped.hip",
     "attn_capped_mfma": "attn_capped_mfma.hip",
+    "attn_normed": "attn_normed.hip",
+    "gated_recurrence": "gated_recurrence.hip",
     "moe": "moe.hip",
     "sampling": "sampling.hip",
     "probe": "probe.hip",

@@ -46,6 +46,7 @@ _PROTOTYPES = {
         "mf_embed_pos": [_P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
         "mf_gelu_tanh": [_P, _P, c_int, c_size_t, _P],
         "mf_weighted_sum": [_P, c_int, c_int, _P, _P, _P, c_int, c_int, _P],
+        "mf_add_rows": [_P, _P, c_size_t, _P],
     },
     "linear_attention": {
         "mf_la_chunk": [],
@@ -57,17 +58,29 @@ _PROTOTYPES = {
         "mf_qkv_conv_prep": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, c_float, _P, _P, _P, c_int, _P, _P, _P,
                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_capped_attn": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_float, c_float, c_int, c_int, c_int, _P],
+                           c_float, c_float, c_int, c_int, _P, _P, c_int, c_int, _P],
         "mf_rope_half_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     },
     "attn_capped_mfma": {
         "mf_capped_mfma": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_int, c_float, c_float, c_int, _P],
+                           c_int, c_float, c_float, c_int, c_int, _P, _P, _P],
+    },
+    "attn_normed": {
+        "mf_qk_norm_prep": [_P, _P, _P, c_float, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, _P, _P, _P,
+                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_unrotate": [_P, c_int, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
+    },
+    "gated_recurrence": {
+        "mf_gr_chunk": [],
+        "mf_gated_scan": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_gated_scan_chunked": [_P, _P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_head_rmsnorm": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float, _P],
     },
     "moe": {
-        "mf_moe_route": [_P, c_int, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
-        "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
-        "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
+        "mf_moe_route": [_P, c_int, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P],
+        "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                          _P],
         "mf_moe_group": [_P, c_int, c_int, _P, _P, _P],
         "mf_moe_gather": [_P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, _P],
         "mf_moe_combine": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
@@ -571,6 +584,152 @@ def weighted_sum(buffers, weights: torch.Tensor, out: torch.Tensor, row_idx: Opt
                                                   _ptr(weights), _ptr(out), rows, d, _stream()), "weighted_sum")
 
 
+def add_rows(h: torch.Tensor, x: torch.Tensor) -> None:
+    """h += x, both float32 of one shape."""
+    _need(h, "add_rows.h", torch.float32)
+    _need(x, "add_rows.x", torch.float32, tuple(h.shape))
+    _check(_fn("elementwise", "mf_add_rows")(_ptr(h), _ptr(x), h.numel(), _stream()), "add_rows")
+
+
+# ------------------------------------------------------------------ gated linear recurrence
+GR_CHUNK = 64            # tokens of a chunk of the chunked form (MF_GR_CHUNK in csrc/gated_recurrence.hip)
+
+
+def gr_chunks(host_new):
+    """The chunk table of the chunked gated recurrence for a step whose sequences bring `host_new` tokens:
+    int32 `[4][n_chunks]` (first token, tokens, sequence, last of its sequence or not) followed by `[n_seqs + 1]`
+    first chunks; and the number of chunks."""
+    t0s, ns, seqs, lasts, firsts = [], [], [], [], [0]
+    t = 0
+    for b, n in enumerate(host_new):
+        for c0 in range(0, n, GR_CHUNK):
+            t0s.append(t + c0)
+            ns.append(min(GR_CHUNK, n - c0))
+            seqs.append(b)
+            lasts.append(1 if c0 + GR_CHUNK >= n else 0)
+        firsts.append(len(t0s))
+        t += n
+    return torch.tensor(t0s + ns + seqs + lasts + firsts, dtype=torch.int32), len(t0s)
+
+
+def gated_scan(proj: torch.Tensor, lower: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Tensor,
+               state: torch.Tensor, out: torch.Tensor, n_heads: int, dim: int, v_dim: int, chunks=None) -> None:
+    """The recurrence S_t = diag(a_t) S_(t-1) + (1 - a_t) v_t^T, o_t = S_t^T silu(q_t), with
+    a_t = lower + (1 - lower) sigmoid(f_t), over a ragged step.  `proj` float32 `[tokens][2 H dim + H v_dim]`:
+    q | f | v; `lower` float32 `[H dim]`; `state` float32 `[slots][H][dim][v_dim]`, read and left at each
+    sequence's last token for the rows `slot_ids`; `out` float32 `[tokens][H v_dim]`.  With `chunks`
+    (`gr_chunks`, the table on the device and its number of chunks) the sequences are walked in chunks side by
+    side."""
+    n_tok = proj.shape[0]
+    n_seqs = slot_ids.numel()
+    _need(proj, "gated_scan.proj", torch.float32, (n_tok, n_heads * (2 * dim + v_dim)))
+    _need(lower, "gated_scan.lower", torch.float32, (n_heads * dim,))
+    _need(cu_seqlens, "gated_scan.cu_seqlens", torch.int32, (n_seqs + 1,))
+    _need(slot_ids, "gated_scan.slot_ids", torch.int32, (n_seqs,))
+    _need(state, "gated_scan.state", torch.float32)
+    if tuple(state.shape[1:]) != (n_heads, dim, v_dim):
+        raise KernelError(f"gated_scan: state {tuple(state.shape)} for {n_heads} heads of {dim} x {v_dim}")
+    _need(out, "gated_scan.out", torch.float32, (n_tok, n_heads * v_dim))
+    if dim > 256:
+        raise KernelError(f"gated_scan: key width {dim} is beyond 256")
+    if chunks is None:
+        _check(_fn("gated_recurrence", "mf_gated_scan")(_ptr(proj), _ptr(lower), _ptr(cu_seqlens), _ptr(slot_ids),
+                                                        _ptr(state), _ptr(out), n_seqs, n_heads, dim, v_dim, _stream()),
+               "gated_scan")
+        return
+    table, n_chunks = chunks
+    _need(table, "gated_scan.chunks", torch.int32, (4 * n_chunks + n_seqs + 1,))
+    per = n_heads * dim * v_dim
+    ws = workspace("gr_chunks", n_chunks * (per + n_heads * dim), proj.device)
+    _check(_fn("gated_recurrence", "mf_gated_scan_chunked")(
+        _ptr(proj), _ptr(lower), _ptr(table), n_chunks, c_void_p(table.data_ptr() + 16 * n_chunks), _ptr(slot_ids),
+        _ptr(state), _ptr(ws), c_void_p(ws.data_ptr() + 4 * n_chunks * per), _ptr(out), n_seqs, n_heads, dim, v_dim,
+        _stream()), "gated_scan_chunked")
+
+
+def head_rmsnorm(o: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor, n_heads: int,
+                 scale: float = 1.0) -> None:
+    """out[t][h] = o[t][h] / sqrt(mean(o[t][h]^2) + eps) * weight * scale: every head of a row normed over its
+    own values, with one gain vector for all heads; o float32 `[tokens][H V]`, out in the run type."""
+    rows, n = o.shape
+    _need(o, "head_rmsnorm.o", torch.float32)
+    if n % n_heads:
+        raise KernelError(f"head_rmsnorm: rows of {n} values are not {n_heads} equal heads")
+    if weight is not None:
+        _need(weight, "head_rmsnorm.weight", torch.float32, (n // n_heads,))
+    _need(out, "head_rmsnorm.out", _FLOATS, (rows, n))
+    _check(_fn("gated_recurrence", "mf_head_rmsnorm")(_ptr(o), _ptr(weight), _ptr(out), _is_bf16(out), rows, n_heads,
+                                                      n // n_heads, float(eps), float(scale), _stream()), "head_rmsnorm")
+
+
+# ------------------------------------------------------------------ normed, pair-rotated queries and keys
+def qk_norm_prep(qkv: torch.Tensor, q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
+                 normed: bool, seq_of_tok: torch.Tensor, positions: torch.Tensor, rot_tables, value_tables,
+                 v_from_k: bool, page_table: torch.Tensor, q_out: torch.Tensor, kcache: torch.Tensor,
+                 vcache: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, v_dim: int,
+                 write_cache: bool = True) -> None:
+    """From the 32-bit q|k|v rows of one product (q|k alone with `v_from_k`): with `normed`, every q and k head
+    over its root mean square (eps inside the root), times `q_gain` / `k_gain` (float32 `[dim]`) where given; the
+    rotation in neighbouring pairs over the first 2 x columns values of a head (`rot_tables` = (cos, sin) or
+    None); the value heads (their own projection, or with `v_from_k` the key heads as projected) rotated in pairs
+    over all their values (`value_tables` = (cos, sin) `[positions][v_dim / 2]` or None); k and v into the cache
+    pages at the tokens' positions and q rounded into `q_out`."""
+    n_tok = positions.numel()
+    C = n_heads * dim + n_kv_heads * dim + (0 if v_from_k else n_kv_heads * v_dim)
+    _need(qkv, "qk_norm_prep.qkv", torch.float32, (n_tok, C))
+    for name, g in (("q_gain", q_gain), ("k_gain", k_gain)):
+        if g is not None:
+            _need(g, "qk_norm_prep." + name, torch.float32, (dim,))
+    rot, cos_r, sin_r = 0, None, None
+    if rot_tables is not None:
+        cos_r, sin_r = rot_tables
+        _need(cos_r, "qk_norm_prep.cos", torch.float32)
+        _need(sin_r, "qk_norm_prep.sin", torch.float32, tuple(cos_r.shape))
+        rot = 2 * cos_r.shape[1]
+        if rot > dim:
+            raise KernelError(f"qk_norm_prep: {rot} rotated values in heads of {dim}")
+    cos_v = sin_v = None
+    if value_tables is not None:
+        cos_v, sin_v = value_tables
+        _need(cos_v, "qk_norm_prep.value cos", torch.float32)
+        _need(sin_v, "qk_norm_prep.value sin", torch.float32, tuple(cos_v.shape))
+        if 2 * cos_v.shape[1] != v_dim:
+            raise KernelError(f"qk_norm_prep: value tables of {cos_v.shape[1]} pairs for values of {v_dim}")
+    if v_from_k and v_dim != dim:
+        raise KernelError(f"qk_norm_prep: values taken from keys of {dim} cannot have {v_dim} values")
+    _need(q_out, "qk_norm_prep.q_out", _FLOATS, (n_tok, n_heads * dim))
+    _need_kv_pages("qk_norm_prep", kcache, vcache, q_out.dtype, n_kv_heads, dim, v_dim)
+    _need(page_table, "qk_norm_prep.page_table", torch.int32)
+    _need(seq_of_tok, "qk_norm_prep.seq_of_tok", torch.int32, (n_tok,))
+    _need(positions, "qk_norm_prep.positions", torch.int32, (n_tok,))
+    _check(_fn("attn_normed", "mf_qk_norm_prep")(
+        _ptr(qkv), _ptr(q_gain), _ptr(k_gain), float(eps), 1 if normed else 0, _ptr(seq_of_tok), _ptr(positions),
+        _ptr(cos_r), _ptr(sin_r), rot, _ptr(cos_v), _ptr(sin_v), 1 if v_from_k else 0, _ptr(page_table),
+        page_table.shape[1], _ptr(q_out), _ptr(kcache), _ptr(vcache), _is_bf16(q_out), n_tok, n_heads, n_kv_heads, dim,
+        v_dim, 1 if write_cache else 0, _stream()), "qk_norm_prep")
+
+
+def unrotate(rows: torch.Tensor, value_tables, positions: torch.Tensor, n_heads: int, scale: float = 1.0) -> None:
+    """Rows `[tokens][H v_dim]` of the run type, in place: pair m of every head turns back by the token's angle m
+    (`value_tables` = (cos, sin) `[positions][v_dim / 2]`; None: no turn), and everything is multiplied by
+    `scale`."""
+    n_tok = positions.numel()
+    _need(rows, "unrotate.rows", _FLOATS)
+    if rows.shape[0] != n_tok or rows.shape[1] % n_heads or (rows.shape[1] // n_heads) % 2:
+        raise KernelError(f"unrotate: rows {tuple(rows.shape)} for {n_tok} tokens of {n_heads} heads")
+    v_dim = rows.shape[1] // n_heads
+    cos_v = sin_v = None
+    if value_tables is not None:
+        cos_v, sin_v = value_tables
+        _need(cos_v, "unrotate.cos", torch.float32)
+        _need(sin_v, "unrotate.sin", torch.float32, tuple(cos_v.shape))
+        if 2 * cos_v.shape[1] != v_dim:
+            raise KernelError(f"unrotate: tables of {cos_v.shape[1]} pairs for values of {v_dim}")
+    _need(positions, "unrotate.positions", torch.int32, (n_tok,))
+    _check(_fn("attn_normed", "mf_unrotate")(_ptr(rows), _is_bf16(rows), _ptr(cos_v), _ptr(sin_v), _ptr(positions), n_tok,
+                                              n_heads, v_dim, float(scale), _stream()), "unrotate")
+
+
 # ------------------------------------------------------------------ linear attention with decay
 LA_CHUNK = 64            # tokens of a chunk of the chunked form (MF_LA_CHUNK in csrc/linear_attention.hip)
 LA_CHUNKED_MAX_DIM = 128  # key width up to which the chunked form's tiles fit into LDS
@@ -723,10 +882,11 @@ def _need_kv_pages(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype,
 def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
                 positions: torch.Tensor, seq_of_tok: torch.Tensor, temp: torch.Tensor, out: torch.Tensor,
                 n_heads: int, n_kv_heads: int, dim: int, v_dim: int, scale: float, cap: float, window: int,
-                max_len: int) -> None:
+                max_len: int, chunk: int = 0, far=None) -> None:
     """Each query token attends to its sequence's cache rows lo..position with
     s = cap tanh(q . k scale temp[head] / cap) (no cap where `cap` is 0), ordinary softmax; keys of
-    `dim` and values of `v_dim` values."""
+    `dim` and values of `v_dim` values.  `chunk`: a token sees only the keys of its own chunk of that many
+    positions, counted from 0.  `far` = (a, b), float32 per head: s -= a[h] ln(1 + b[h] (position - key))."""
     n_tok = positions.numel()
     _need(q, "capped_attn.q", _FLOATS, (n_tok, n_heads * dim))
     _need(out, "capped_attn.out", q.dtype, (n_tok, n_heads * v_dim))
@@ -740,9 +900,12 @@ def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
                           f"{v_dim} (at most 256)")
     if max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"capped_attn: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
+    far_a, far_b = _far_pair("capped_attn", far, n_heads)
     # keys split over workgroups where tokens x kv heads alone do not fill the chip: at least 256 keys a split;
     # a windowed token's splits start at its window's first key
     reach = min(max_len, window) if window else max_len
+    if chunk:
+        reach = min(reach, int(chunk))
     blocks = n_tok * n_kv_heads * ((n_heads // n_kv_heads + 7) // 8)
     n_splits = max(1, min(1024 // max(1, blocks), (reach + 255) // 256, 64))
     split_len = ((reach + n_splits - 1) // n_splits + PAGE - 1) // PAGE * PAGE
@@ -751,7 +914,18 @@ def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
     _check(_fn("attn_capped", "mf_capped_attn")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(seq_of_tok),
         _ptr(temp), _ptr(out), _ptr(part), _is_bf16(q), n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale),
-        float(cap or 0.0), int(window or 0), n_splits, split_len, _stream()), "capped_attn")
+        float(cap or 0.0), int(window or 0), int(chunk or 0), _ptr(far_a), _ptr(far_b), n_splits, split_len, _stream()),
+        "capped_attn")
+
+
+def _far_pair(what: str, far, n_heads: int):
+    """The two per-head vectors of the penalty on distance, checked; (None, None) without one."""
+    if far is None:
+        return None, None
+    a, b = far
+    _need(a, what + ".far[0]", torch.float32, (n_heads,))
+    _need(b, what + ".far[1]", torch.float32, (n_heads,))
+    return a, b
 
 
 CAPPED_MFMA_ROWS = 16        # consecutive tokens of a sequence that a wave of the matrix-core form takes
@@ -764,7 +938,7 @@ def capped_mfma_takes(dtype, dim: int, v_dim: int) -> bool:
 
 def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor, ctx,
                         temp: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, v_dim: int,
-                        scale: float, cap: float, window: int) -> None:
+                        scale: float, cap: float, window: int, chunk: int = 0, far=None) -> None:
     """`capped_attn` in bfloat16 on the matrix cores: blocks of 16 consecutive new tokens of a sequence
     (`ctx.query_tiles`) times the query heads of a kv head.  A decode step (one token a sequence) splits every
     token's keys over several waves (at least 128 keys a split) and merges the parts in their order."""
@@ -783,12 +957,15 @@ def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Ten
         raise KernelError(f"capped_attn_prefill: {n_heads} heads over {n_kv_heads} kv heads")
     if ctx.max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"capped_attn_prefill: max_len {ctx.max_len} exceeds the page table")
+    far_a, far_b = _far_pair("capped_attn_prefill", far, n_heads)
     n_splits, split_len, part = 1, 0, None
     if ctx.all_decode:
         # every sequence is a tile of one token; nothing comes from the host (the step may be captured)
         tile_seq = ctx.seq_of_tok
         tile_q0 = torch.zeros(n_tok, dtype=torch.int32, device=q.device)
         reach = min(ctx.max_len, window) if window else ctx.max_len
+        if chunk:
+            reach = min(reach, int(chunk))
         waves = n_tok * n_kv_heads * max(1, (n_heads // n_kv_heads) // 2)
         n_splits = max(1, min(4 * cu_count() // max(1, waves), (reach + 31 + 127) // 128, 64))
         split_len = (((reach + 31 + n_splits - 1) // n_splits) + 31) // 32 * 32
@@ -801,7 +978,8 @@ def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Ten
     _check(_fn("attn_capped_mfma", "mf_capped_mfma", lib)(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
         _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), tile_seq.numel(), _ptr(temp), _ptr(out), _ptr(part), n_splits,
-        split_len, n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale), float(cap or 0.0), int(window or 0), _stream()),
+        split_len, n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale), float(cap or 0.0), int(window or 0),
+        int(chunk or 0), _ptr(far_a), _ptr(far_b), _stream()),
         "capped_attn_decode" if ctx.all_decode else "capped_attn_prefill")
 
 
@@ -811,12 +989,13 @@ MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128     # what `moe_sparse` takes in o
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, dense: Optional[torch.Tensor], chosen: torch.Tensor,
-              weights: torch.Tensor, n_groups: int, keep: int) -> None:
+              weights: torch.Tensor, n_groups: int, keep: int, bias: Optional[torch.Tensor] = None) -> None:
     """The router: logits = router x in 32-bit (`router` float32 `[experts][K]`, `x` `[tokens][K]` in the run
     type), softmax scores, the `keep` best of `n_groups` groups of neighbouring experts (a group's score is
     its best expert's), the `chosen.shape[1]` best experts of those groups, weighted by their scores over
     their sum.  `dense` `[tokens][experts]`, where given, gets the weights at the chosen experts and 0
-    elsewhere; `chosen`, `weights` `[tokens][top]`."""
+    elsewhere; `chosen`, `weights` `[tokens][top]`.  `bias` float32 `[experts]` is added to the logits.  With one
+    group the weights are the softmax over the chosen logits alone."""
     n_tok, K = x.shape
     E = router.shape[0]
     top = chosen.shape[1]
@@ -828,13 +1007,19 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, dense: Optional[torch.Tenso
     _need(weights, "moe_route.weights", torch.float32, (n_tok, top))
     if E > MOE_MAX_EXPERTS or E % n_groups or not 1 <= keep <= n_groups or not 1 <= top <= min(64, keep * (E // n_groups)):
         raise KernelError(f"moe_route: {E} experts in {n_groups} groups, {keep} kept, {top} chosen")
-    _check(_fn("moe", "mf_moe_route")(_ptr(x), _is_bf16(x), _ptr(router), K, _ptr(dense), _ptr(chosen), _ptr(weights),
+    if bias is not None:
+        _need(bias, "moe_route.bias", torch.float32, (E,))
+    _check(_fn("moe", "mf_moe_route")(_ptr(x), _is_bf16(x), _ptr(router), _ptr(bias), K, _ptr(dense), _ptr(chosen), _ptr(weights),
                                        n_tok, E, n_groups, keep, top, _stream()), "moe_route")
 
 
-def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: float) -> None:
+MOE_ACTS = {"clamped_swish": 0, "silu": 1}      # the experts' activations (MF_MOE_ACT_* in csrc/moe.hip)
+
+
+def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: float, act: int = 0) -> None:
     """`gu` float32 `[tokens][experts][2 F]` (gate sums, then up sums): out `[tokens][experts F]` =
-    dense[t][e] g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    dense[t][e] g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); with `act` 1,
+    dense[t][e] silu(gate) up."""
     n_tok, E = dense.shape
     _need(dense, "moe_act.dense", torch.float32)
     _need(gu, "moe_act.gu", torch.float32)
@@ -843,11 +1028,11 @@ def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: flo
     F = gu.shape[1] // (2 * E)
     _need(out, "moe_act.out", _FLOATS, (n_tok, E * F))
     _check(_fn("moe", "mf_moe_act")(_ptr(gu), _ptr(dense), _ptr(out), _is_bf16(out), n_tok, E, F, float(limit),
-                                     _stream()), "moe_act")
+                                     int(act), _stream()), "moe_act")
 
 
 def moe_sparse(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
-               out: torch.Tensor, n_experts: int, limit: float) -> None:
+               out: torch.Tensor, n_experts: int, limit: float, act: int = 0) -> None:
     """The chosen experts only, for steps of few tokens: `gate_up` `[experts][2 F][K]` (an expert's gate
     rows, then its up rows), `down` `[experts][N][F]`; out `[tokens][N]` float32 += the weighted sum of the
     chosen experts' outputs, choices added in their order."""
@@ -866,7 +1051,7 @@ def moe_sparse(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chose
     y = torch.empty((n_tok, top, F), dtype=x.dtype, device=x.device)
     rows = torch.empty((n_tok * top, N), dtype=torch.float32, device=x.device)
     _check(_fn("moe", "mf_moe_sparse")(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(y), _ptr(rows), _ptr(out),
-                                        _is_bf16(x), n_tok, top, n_experts, F, K, N, float(limit), _stream()), "moe_sparse")
+                                        _is_bf16(x), n_tok, top, n_experts, F, K, N, float(limit), int(act), _stream()), "moe_sparse")
 
 SCAN_CHUNK = 32          # tokens of a chunk of the chunked scan (MF_SCAN_CHUNK in csrc/recurrence.hip)
 

@@ -120,6 +120,41 @@ class BranchNormBlock(Block):
         return h
 
 
+@register_block("sandwich")
+class SandwichBlock(BranchNormBlock):
+    """h += N1b(mixer(N1(h))); h += N2b(feed_forward(N2(h))): a norm before every branch and one behind it, on
+    the way into the stream.  norms: "mixer" and "mixer_out" around the mixer, "feed_forward" and
+    "feed_forward_out" around the feed-forward; a block without one branch has neither that branch nor its two
+    norms.  The norm before a branch may stay lazy (folded into the branch's first product); the one behind it
+    adds into the stream in the same kernel."""
+
+    optional_norms = ("mixer", "mixer_out", "feed_forward", "feed_forward_out")
+
+    def __init__(self, mixer, feed_forward, norms, rt):
+        Block.__init__(self, mixer, feed_forward, norms, rt)
+        for part, names in ((mixer, ("mixer", "mixer_out")), (feed_forward, ("feed_forward", "feed_forward_out"))):
+            for name in names:
+                if (part is None) != (name not in self.norms):
+                    raise ValueError(f"sandwich block: a branch and the norms around it come together or not at all "
+                                     f"({name!r})")
+
+    def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
+        ctx.norm_next = ctx.norm_ahead = None
+        if self.mixer is not None:
+            x = normed_input(self.norms["mixer"], self.mixer, h)
+            y = self._run(self.mixer, x, h.shape[0], h.shape[1], ctx, entry, writes_cache)
+            self.norms["mixer_out"].add_normed(y, h)
+        if keep_rows is not None:
+            kept = torch.empty((keep_rows.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
+            ops.gather_rows(h, keep_rows, kept)
+            h = kept
+        if self.feed_forward is not None:
+            x = normed_input(self.norms["feed_forward"], self.feed_forward, h)
+            y = self._run(self.feed_forward, x, h.shape[0], h.shape[1], ctx)
+            self.norms["feed_forward_out"].add_normed(y, h)
+        return h
+
+
 @register_block("parallel")
 class ParallelBlock(Block):
     """x + mixer(N1(x)) + feed_forward(N2(x)): both branches read the same x, each through a norm of

@@ -3,8 +3,11 @@
 Router: z = Wr x in 32-bit, scores = softmax(z) over all experts; the experts form `groups` equal
 groups of neighbours, a group's score is its best expert's, and only experts of the `keep` best groups
 can be among the `top` chosen; the chosen experts' scores over their sum are the weights.
+With one group (and so all of it kept) the weights are the softmax over the chosen logits alone.  A router may
+add a bias per expert to its logits.
 Expert (no biases): g = min(Wg x, limit), u = clamp(Wu x, -limit, limit), y = g sigmoid(1.702 g) (u + 1),
-output Wd y.  The result is the weighted sum of the chosen experts' outputs.
+output Wd y; or, with `act` "silu", the plain gated form y = silu(Wg x) (Wu x).  The result is the weighted sum
+of the chosen experts' outputs.
 
 Two forms, both of which read or multiply only what was chosen.  Steps of few tokens and decode steps (which
 may be captured, so nothing may wait for the host): `ops.moe_sparse`, up to 16 tokens a launch, reads every
@@ -31,8 +34,9 @@ SPARSE_UP_TO = ops.MOE_SPARSE_TOKENS
 
 @register_feed_forward("grouped_moe")
 class GroupedMoE(FeedForward):
-    """params: hidden_size, intermediate_size (of one expert), n_experts, top, groups, keep, limit,
-    router (tensor name), expert (format of an expert's tensor stem, e.g. "mlp.e{}"; its matrices are
+    """params: hidden_size, intermediate_size (of one expert), n_experts, top, groups and keep (default 1: no
+    groups), act ("clamped_swish", the default, with `limit`; or "silu"), router (tensor name), router_bias
+    (tensor name, or None), expert (format of an expert's tensor stem, e.g. "mlp.e{}"; its matrices are
     stem + ".gate", ".up", ".down")."""
 
     can_overwrite = True
@@ -40,18 +44,26 @@ class GroupedMoE(FeedForward):
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         p = spec.params
-        self.hidden, self.inter, self.ne, self.top, self.groups, self.keep = (
-            int(p[k]) for k in ("hidden_size", "intermediate_size", "n_experts", "top", "groups", "keep"))
-        self.limit = float(p["limit"])
+        self.hidden, self.inter, self.ne, self.top = (
+            int(p[k]) for k in ("hidden_size", "intermediate_size", "n_experts", "top"))
+        self.groups, self.keep = int(p.get("groups", 1)), int(p.get("keep", p.get("groups", 1)))
+        act = p.get("act", "clamped_swish")
+        if act not in ops.MOE_ACTS:
+            raise ValueError(f"grouped_moe: activation {act!r} is not one of {sorted(ops.MOE_ACTS)}")
+        self.act = ops.MOE_ACTS[act]
+        self.limit = float(p["limit"]) if act == "clamped_swish" else 0.0
         self.router_name, self.expert_name = p["router"], p["expert"]
+        self.bias_name = p.get("router_bias")
         per = self.ne // max(1, self.groups)
         if self.ne % self.groups or not 1 <= self.keep <= self.groups or not 1 <= self.top <= min(64, self.keep * per) \
                 or self.ne > ops.MOE_MAX_EXPERTS:
             raise ValueError(f"grouped_moe: {self.ne} experts in {self.groups} groups, {self.keep} kept, {self.top} chosen")
-        self.router = self.gate_up = self.down = None
+        self.router = self.router_bias = self.gate_up = self.down = None
 
     def tensor_specs(self):
         s = {self.router_name: TensorSpec((self.ne, self.hidden))}
+        if self.bias_name is not None:
+            s[self.bias_name] = TensorSpec((self.ne,))
         for e in range(self.ne):
             stem = self.expert_name.format(e)
             s[stem + ".gate"] = TensorSpec((self.inter, self.hidden))
@@ -61,6 +73,8 @@ class GroupedMoE(FeedForward):
 
     def load(self, get):
         self.router = get(self.router_name).to(torch.float32).contiguous()   # the router's product is 32-bit
+        if self.bias_name is not None:
+            self.router_bias = get(self.bias_name).to(torch.float32).contiguous()
         stems = [self.expert_name.format(e) for e in range(self.ne)]
         # [experts][gate | up][hidden] and [experts][hidden][inter]: an expert's matrices are contiguous slices
         self.gate_up = torch.stack([torch.cat([get(s + ".gate"), get(s + ".up")], dim=0) for s in stems]).contiguous()
@@ -74,7 +88,7 @@ class GroupedMoE(FeedForward):
         n, dev = x.shape[0], x.device
         chosen = torch.empty((n, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((n, self.top), dtype=torch.float32, device=dev)
-        ops.moe_route(x, self.router, None, chosen, weights, self.groups, self.keep)
+        ops.moe_route(x, self.router, None, chosen, weights, self.groups, self.keep, bias=self.router_bias)
         log = ctx._memo.get("route_log") if ctx is not None else None
         if log is not None:                  # a caller that wants to know: every routed layer's choices, in run order
             log.append(chosen)
@@ -86,7 +100,7 @@ class GroupedMoE(FeedForward):
                 h.zero_()
             for t0 in range(0, n, few):      # (slices of a contiguous tensor's rows are contiguous)
                 ops.moe_sparse(x[t0:t0 + few], self.gate_up, self.down, chosen[t0:t0 + few], weights[t0:t0 + few],
-                               h[t0:t0 + few], self.ne, self.limit)
+                               h[t0:t0 + few], self.ne, self.limit, self.act)
             return
         rank = torch.empty_like(chosen)
         counts = torch.empty(self.ne, dtype=torch.int32, device=dev)
@@ -104,7 +118,7 @@ class GroupedMoE(FeedForward):
             if per_expert[e]:
                 gate_up(xs[starts[e]:starts[e + 1]], out=gu[starts[e]:starts[e + 1]])
         y = torch.empty((pairs, self.inter), dtype=self.rt.dtype, device=dev)
-        ops.moe_act(gu, self._ones(pairs, dev), y, self.limit)
+        ops.moe_act(gu, self._ones(pairs, dev), y, self.limit, self.act)
         rows = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
         for e, (_, down) in enumerate(self.experts):
             if per_expert[e]:

@@ -10,6 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import TensorSpec
 from .base import Norm, register_norm
+from .spec import PartSpec
 
 
 @register_norm("rmsnorm")
@@ -86,3 +87,19 @@ class ScalarRMSNorm(RMSNorm):
     def load(self, get):
         g = get(self.name).to(torch.float32).reshape(1)
         self.weight = g.expand(self.size).contiguous()
+
+
+@register_norm("offset_rmsnorm")
+class OffsetRMSNorm(GroupRMSNorm):
+    """RMS norm whose weight is stored around zero: x / sqrt(mean(x^2) + eps) * (1 + w).  The gain 1 + w is
+    formed once, in 32-bit, when the weights arrive, so every kernel and fold of the plain norm serves it,
+    also the one that adds a normed branch result into the stream.  params: size, eps, weight (tensor name)."""
+
+    def __init__(self, spec, rt):
+        super().__init__(PartSpec(spec.kind, dict(spec.params, groups=1)), rt)
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.size,), init="zeros")}
+
+    def load(self, get):
+        self.weight = (get(self.name).to(torch.float32) + 1.0).contiguous()

@@ -60,10 +60,13 @@ class RunEntry:
     """One position of the run order.  `block` indexes `ModelSpec.blocks` and may appear
     in several entries.  `cache` is the cache entry the mixer uses; entries that name the
     same `cache` share keys and values, and only the entry with `writes_cache` stores
-    into it (the other reads what the first one wrote in the same step)."""
+    into it (the other reads what the first one wrote in the same step).  With `adds_embedding` the
+    embedding output of the step's tokens is added to the stream right before the block runs (a run of
+    blocks that is passed again takes its input in anew)."""
     block: int
     cache: int
     writes_cache: bool = True
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)

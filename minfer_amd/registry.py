@@ -46,6 +46,8 @@ def _register_builtin() -> None:
     register_architecture(tabezen.ARCHITECTURE, tabezen.TabezenConfig)
     from .config import lagedra
     register_architecture(lagedra.ARCHITECTURE, lagedra.LagedraConfig)
+    from .config import nodutar
+    register_architecture(nodutar.ARCHITECTURE, nodutar.NodutarConfig)
 
 
 _register_builtin()

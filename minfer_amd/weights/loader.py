@@ -26,7 +26,8 @@ class WeightError(ValueError):
 @dataclass(frozen=True)
 class TensorSpec:
     """What a part expects of one tensor: its shape, and how random weights fill it
-    ('normal': N(0, std) of the configuration; 'ones': norm gains)."""
+    ('normal': N(0, std) of the configuration; 'ones': norm gains; 'zeros': gains stored around
+    zero; 'halves': bounds that lie between 0 and 1)."""
     shape: Tuple[int, ...]
     init: str = "normal"
 

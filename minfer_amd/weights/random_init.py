@@ -37,6 +37,8 @@ def random_tensor(seed: int, name: str, spec: TensorSpec, std: float,
         return torch.ones(spec.shape, dtype=dtype)
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=dtype)
+    if spec.init == "halves":
+        return torch.full(spec.shape, 0.5, dtype=dtype)
     if spec.init != "normal":
         raise ValueError(f"{name}: unknown init {spec.init!r}")
     if dtype not in (torch.bfloat16, torch.float32):

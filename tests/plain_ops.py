@@ -450,13 +450,15 @@ def qkv_conv_prep(qkv, conv_w, conv_state, cu_seqlens, seq_of_tok, slot_ids, pos
 
 
 def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out, n_heads, n_kv_heads, dim, v_dim,
-                scale, cap, window, max_len):
+                scale, cap, window, max_len, chunk=0, far=None):
     t_all = positions.numel()
     group = n_heads // n_kv_heads
     qq = q.double().view(t_all, n_heads, dim)
     for i in range(t_all):
         p = int(positions[i])
         lo = max(0, p - window + 1) if window else 0
+        if chunk:
+            lo = max(lo, p // chunk * chunk)
         pos = torch.arange(lo, p + 1)
         pages = page_table[int(seq_of_tok[i])].long()[pos // PAGE]
         assert (pages >= 0).all(), "attention reads a page that was given back"
@@ -467,6 +469,8 @@ def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out,
             s = (keys @ qq[i, h]) * scale * float(temp[h])
             if cap:
                 s = cap * torch.tanh(s / cap)
+            if far is not None:
+                s = s - float(far[0][h]) * torch.log1p(float(far[1][h]) * (p - pos).double())
             out[i, h * v_dim:(h + 1) * v_dim] = (torch.softmax(s, dim=0) @ vals).to(out.dtype)
 
 
@@ -474,9 +478,92 @@ def capped_mfma_takes(dtype, dim, v_dim):
     return dtype == torch.bfloat16 and dim % 16 == 0 and v_dim % 16 == 0 and 16 <= dim <= 256 and 16 <= v_dim <= 256
 
 
-def capped_attn_prefill(q, kcache, vcache, page_table, ctx, temp, out, n_heads, n_kv_heads, dim, v_dim, scale, cap, window):
+def capped_attn_prefill(q, kcache, vcache, page_table, ctx, temp, out, n_heads, n_kv_heads, dim, v_dim, scale, cap, window,
+                        chunk=0, far=None):
     capped_attn(q, kcache, vcache, page_table, ctx.positions, ctx.seq_of_tok, temp, out, n_heads, n_kv_heads, dim, v_dim,
-                scale, cap, window, ctx.max_len)
+                scale, cap, window, ctx.max_len, chunk=chunk, far=far)
+
+
+# ------------------------------------------------------------------ rows added into rows, the gated recurrence,
+# normed and pair-rotated queries and keys
+def add_rows(h, x):
+    h.add_(x)
+
+
+GR_CHUNK = 64
+
+
+def gr_chunks(host_new):
+    return torch.zeros(0, dtype=torch.int32), 0
+
+
+def gated_scan(proj, lower, cu_seqlens, slot_ids, state, out, n_heads, dim, v_dim, chunks=None):
+    H, D, V = n_heads, dim, v_dim
+    p = proj.double()
+    low = lower.double().view(H, D)
+    for b in range(slot_ids.numel()):
+        r0, r1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
+        slot = int(slot_ids[b])
+        S = state[slot].double()
+        for t in range(r0, r1):
+            z = p[t, :H * D].view(H, D)
+            q = z * torch.sigmoid(z)
+            a = low + (1.0 - low) * torch.sigmoid(p[t, H * D:2 * H * D].view(H, D))
+            v = p[t, 2 * H * D:].view(H, V)
+            S = a[:, :, None] * S + (1.0 - a)[:, :, None] * v[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, q).reshape(-1).float()
+        state[slot] = S.float()
+
+
+def head_rmsnorm(o, weight, eps, out, n_heads, scale=1.0):
+    rows, n = o.shape
+    x = o.double().view(rows, n_heads, n // n_heads)
+    y = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * scale
+    if weight is not None:
+        y = y * weight.double()
+    out.copy_(y.reshape(rows, n).to(out.dtype))
+
+
+def qk_norm_prep(qkv, q_gain, k_gain, eps, normed, seq_of_tok, positions, rot_tables, value_tables, v_from_k, page_table,
+                 q_out, kcache, vcache, n_heads, n_kv_heads, dim, v_dim, write_cache=True):
+    t_all = positions.numel()
+    y = qkv.double()
+    nq, nk = n_heads * dim, n_kv_heads * dim
+    q = y[:, :nq].view(t_all, n_heads, dim)
+    k = y[:, nq:nq + nk].view(t_all, n_kv_heads, dim)
+    v = k.clone() if v_from_k else y[:, nq + nk:].view(t_all, n_kv_heads, v_dim)
+    if normed:
+        q = q / torch.sqrt((q * q).mean(dim=-1, keepdim=True) + eps)
+        k = k / torch.sqrt((k * k).mean(dim=-1, keepdim=True) + eps)
+    if q_gain is not None:
+        q = q * q_gain.double()
+    if k_gain is not None:
+        k = k * k_gain.double()
+    pos = positions.long()
+    if rot_tables is not None:
+        c, s = rot_tables[0][pos].double()[:, None, :], rot_tables[1][pos].double()[:, None, :]
+        q, k = _rotate_pairs(q, c, s), _rotate_pairs(k, c, s)
+    if value_tables is not None:
+        v = _rotate_pairs(v, value_tables[0][pos].double()[:, None, :], value_tables[1][pos].double()[:, None, :])
+    q_out.copy_(q.reshape(t_all, nq).to(q_out.dtype))
+    if not write_cache:
+        return
+    for i in range(t_all):
+        p = int(positions[i])
+        page = int(page_table[int(seq_of_tok[i]), p // PAGE])
+        assert page >= 0
+        kcache[page, :, p % PAGE] = k[i].to(kcache.dtype)
+        for g in range(n_kv_heads):
+            _store_v(vcache, page, p % PAGE, g, v[i, g])
+
+
+def unrotate(rows, value_tables, positions, n_heads, scale=1.0):
+    t_all = positions.numel()
+    x = rows.double().view(t_all, n_heads, -1)
+    if value_tables is not None:
+        pos = positions.long()
+        x = _rotate_pairs(x, value_tables[0][pos].double()[:, None, :], -value_tables[1][pos].double()[:, None, :])
+    rows.copy_((x * scale).reshape(t_all, -1).to(rows.dtype))
 
 
 # ------------------------------------------------------------------ mixture of experts
@@ -484,8 +571,14 @@ MOE_MAX_EXPERTS = 1024
 MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128
 
 
-def moe_route(x, router, dense, chosen, weights, n_groups, keep):
-    logits = (x.double() @ router.double().t()).float()
+MOE_ACTS = {"clamped_swish": 0, "silu": 1}
+
+
+def moe_route(x, router, dense, chosen, weights, n_groups, keep, bias=None):
+    logits = x.double() @ router.double().t()
+    if bias is not None:
+        logits = logits + bias.double()
+    logits = logits.float()
     n_tok, E = logits.shape
     top = chosen.shape[1]
     per = E // n_groups
@@ -506,21 +599,23 @@ def moe_route(x, router, dense, chosen, weights, n_groups, keep):
             dense[t, pick] = w
 
 
-def _expert_act(g, u, limit):
+def _expert_act(g, u, limit, act=0):
+    if act == 1:
+        return g * torch.sigmoid(g) * u
     g = torch.clamp(g, max=limit)
     u = torch.clamp(u, -limit, limit)
     return g * torch.sigmoid(1.702 * g) * (u + 1.0)
 
 
-def moe_act(gu, dense, out, limit):
+def moe_act(gu, dense, out, limit, act=0):
     n_tok, E = dense.shape
     F = gu.shape[1] // (2 * E)
     x = gu.double().view(n_tok, E, 2, F)
-    y = _expert_act(x[:, :, 0], x[:, :, 1], limit) * dense.double()[:, :, None]
+    y = _expert_act(x[:, :, 0], x[:, :, 1], limit, act) * dense.double()[:, :, None]
     out.copy_(y.reshape(n_tok, E * F).to(out.dtype))
 
 
-def moe_sparse(x, gate_up, down, chosen, weights, out, n_experts, limit):
+def moe_sparse(x, gate_up, down, chosen, weights, out, n_experts, limit, act=0):
     n_tok, K = x.shape
     _, N, F = down.shape
     gu = gate_up.double().view(n_experts, 2, F, K)
@@ -528,7 +623,7 @@ def moe_sparse(x, gate_up, down, chosen, weights, out, n_experts, limit):
     for t in range(n_tok):
         for k in range(chosen.shape[1]):
             e = int(chosen[t, k])
-            y = _expert_act(gu[e, 0] @ x[t].double(), gu[e, 1] @ x[t].double(), limit).to(x.dtype).double()
+            y = _expert_act(gu[e, 0] @ x[t].double(), gu[e, 1] @ x[t].double(), limit, act).to(x.dtype).double()
             out[t] += (float(weights[t, k]) * (dn[e] @ y)).float()
 
 
@@ -632,7 +727,8 @@ NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", 
          "group_rmsnorm", "xielu", "rope_table_freqs", "rope_pairs_inplace", "mingru_scan", "latent_prep",
          "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma",
          "embed_pos", "gelu_tanh", "weighted_sum", "lightning_scan", "gated_rmsnorm", "rope_half_inplace",
-         "qkv_conv_prep", "capped_attn", "capped_mfma_takes", "capped_attn_prefill", "moe_route", "moe_act", "moe_sparse", "moe_group", "moe_gather", "moe_combine"]
+         "qkv_conv_prep", "capped_attn", "capped_mfma_takes", "capped_attn_prefill", "moe_route", "moe_act", "moe_sparse", "moe_group", "moe_gather", "moe_combine",
+         "add_rows", "gr_chunks", "gated_scan", "head_rmsnorm", "qk_norm_prep", "unrotate"]
 
 
 def install(monkeypatch):
