@@ -99,11 +99,15 @@ def route(h, router, bias, top: int):
     return chosen, softmax(picked)
 
 
-def moe(h, w, prefix: str, n_experts: int, top: int, forced=None):
+def moe(h, w, prefix: str, n_experts: int, top: int, forced=None, margins=None):
     """`forced`: the choices to take instead of the router's own (the weights are still the softmax of
-    the chosen logits)."""
+    the chosen logits).  `margins`, a list, gets per token the gap between the last logit chosen and the
+    first one left out (infinite where all experts are chosen)."""
     z = h @ w[prefix + "router"].T + w[prefix + "router.b"]
     chosen, weights = route(h, w[prefix + "router"], w[prefix + "router.b"], top)
+    if margins is not None:
+        ranked = -np.sort(-z, axis=-1)
+        margins.append(ranked[:, top - 1] - ranked[:, top] if top < n_experts else np.full(h.shape[0], np.inf))
     if forced is not None:
         chosen = np.asarray(forced)
         weights = softmax(np.take_along_axis(z, chosen, axis=-1))
@@ -202,7 +206,7 @@ def run_order(cfg):
     return order + [(i, False) for i in range(loop["stop"], n)]
 
 
-def forward(cfg, w, tokens, forced=None, keep_layers: bool = False):
+def forward(cfg, w, tokens, forced=None, keep_layers: bool = False, margins=None):
     """Logits [tokens][vocab] of one whole sequence from position 0.  `forced`: per run of a layer with a
     feed-forward, the experts to take (None: the router's own).  Returns (logits, streams after every
     layer run, choices per routed layer run)."""
@@ -226,7 +230,7 @@ def forward(cfg, w, tokens, forced=None, keep_layers: bool = False):
         if layer.get("mlp") is not None:
             r = layer["mlp"]["router"]
             f = None if forced is None else forced[len(choices)]
-            y, chosen = moe(offset_norm(x, w[p + "norm2"], eps), w, p + "mlp.", r["experts"], r["top"], f)
+            y, chosen = moe(offset_norm(x, w[p + "norm2"], eps), w, p + "mlp.", r["experts"], r["top"], f, margins)
             choices.append(chosen)
             x = x + offset_norm(y, w[p + "norm2b"], eps)
         if keep_layers:
@@ -239,3 +243,32 @@ def load(folder: str):
     with open(os.path.join(folder, "config.json")) as f:
         cfg = json.load(f)
     return cfg, read_safetensors(os.path.join(folder, "model.safetensors"))
+
+
+def greedy(row) -> int:
+    return int(np.argmax(row))
+
+
+class PlainNodutar:
+    def __init__(self, cfg, w):
+        self.cfg, self.w = cfg, w
+
+    @classmethod
+    def from_folder(cls, folder: str):
+        return cls(*load(folder))
+
+    def routed_runs(self):
+        """The runs of layers (positions of the run order) that have a feed-forward."""
+        return [n for n, (i, _) in enumerate(run_order(self.cfg)) if self.cfg["layers"][i].get("mlp") is not None]
+
+    def forward(self, tokens, routes=None, margins=None, choices=None):
+        """Logits [tokens][vocab].  `routes`: {run: [tokens][top]} experts to take; `margins` and `choices`
+        (lists) get the routers' margins and own choices per routed run."""
+        forced = None if routes is None else [routes[n] for n in self.routed_runs()]
+        logits, _, own = forward(self.cfg, self.w, tokens, forced=forced, margins=margins)
+        if choices is not None:
+            if routes is None:
+                choices.extend(own)
+            else:                                 # the router's own choices, not the forced ones
+                choices.extend(forward(self.cfg, self.w, tokens)[2])
+        return logits
