@@ -162,9 +162,10 @@ class DecodeSession:
         windowed = any(g.request.gives_pages_back for g in cache.groups)
         if grows:
             cache.reserve({s: new_len[s] for s in grows})
-        if grows or windowed or not self._host_tables:
+        fresh = not self._host_tables        # just bound: every group's rows are due
+        if grows or windowed or fresh:
             for g in cache.groups:
-                if self._host_tables and not grows and not g.request.gives_pages_back:
+                if not fresh and not grows and not g.request.gives_pages_back:
                     continue
                 rows = cache.page_rows(g, self.slots, self.n_cols)
                 if self._host_tables.get(id(g)) != rows:

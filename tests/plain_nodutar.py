@@ -99,15 +99,17 @@ def route(h, router, bias, top: int):
     return chosen, softmax(picked)
 
 
-def moe(h, w, prefix: str, n_experts: int, top: int, forced=None, margins=None):
+def moe(h, w, prefix: str, n_experts: int, top: int, forced=None, margins=None, own=None):
     """`forced`: the choices to take instead of the router's own (the weights are still the softmax of
     the chosen logits).  `margins`, a list, gets per token the gap between the last logit chosen and the
-    first one left out (infinite where all experts are chosen)."""
+    first one left out (infinite where all experts are chosen); `own`, a list, the router's own choices."""
     z = h @ w[prefix + "router"].T + w[prefix + "router.b"]
     chosen, weights = route(h, w[prefix + "router"], w[prefix + "router.b"], top)
     if margins is not None:
         ranked = -np.sort(-z, axis=-1)
         margins.append(ranked[:, top - 1] - ranked[:, top] if top < n_experts else np.full(h.shape[0], np.inf))
+    if own is not None:
+        own.append(chosen)
     if forced is not None:
         chosen = np.asarray(forced)
         weights = softmax(np.take_along_axis(z, chosen, axis=-1))
@@ -206,10 +208,11 @@ def run_order(cfg):
     return order + [(i, False) for i in range(loop["stop"], n)]
 
 
-def forward(cfg, w, tokens, forced=None, keep_layers: bool = False, margins=None):
+def forward(cfg, w, tokens, forced=None, keep_layers: bool = False, margins=None, own=None):
     """Logits [tokens][vocab] of one whole sequence from position 0.  `forced`: per run of a layer with a
     feed-forward, the experts to take (None: the router's own).  Returns (logits, streams after every
-    layer run, choices per routed layer run)."""
+    layer run, choices taken per routed layer run).  `own` (a list) gets what every router would have
+    chosen itself, given what was taken before it."""
     eps = cfg["norm"]["eps"]
     x = w["embed"][np.asarray(tokens)]
     first = x.copy()
@@ -230,7 +233,7 @@ def forward(cfg, w, tokens, forced=None, keep_layers: bool = False, margins=None
         if layer.get("mlp") is not None:
             r = layer["mlp"]["router"]
             f = None if forced is None else forced[len(choices)]
-            y, chosen = moe(offset_norm(x, w[p + "norm2"], eps), w, p + "mlp.", r["experts"], r["top"], f, margins)
+            y, chosen = moe(offset_norm(x, w[p + "norm2"], eps), w, p + "mlp.", r["experts"], r["top"], f, margins, own)
             choices.append(chosen)
             x = x + offset_norm(y, w[p + "norm2b"], eps)
         if keep_layers:
@@ -263,12 +266,11 @@ class PlainNodutar:
 
     def forward(self, tokens, routes=None, margins=None, choices=None):
         """Logits [tokens][vocab].  `routes`: {run: [tokens][top]} experts to take; `margins` and `choices`
-        (lists) get the routers' margins and own choices per routed run."""
+        (lists) get, per routed run, the routers' margins and what they would have chosen themselves given
+        the choices taken before them."""
         forced = None if routes is None else [routes[n] for n in self.routed_runs()]
-        logits, _, own = forward(self.cfg, self.w, tokens, forced=forced, margins=margins)
+        own = []
+        logits, _, _ = forward(self.cfg, self.w, tokens, forced=forced, margins=margins, own=own)
         if choices is not None:
-            if routes is None:
-                choices.extend(own)
-            else:                                 # the router's own choices, not the forced ones
-                choices.extend(forward(self.cfg, self.w, tokens)[2])
+            choices.extend(own)
         return logits

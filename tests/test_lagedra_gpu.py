@@ -14,10 +14,11 @@ import plain_lagedra as pl
 import plain_ops
 from lagedra_tiny import LG, LG_A, LG_C, attention, dense, random_config, write_lagedra
 from replays import batch_steps, chunk_steps, requests_for, run_steps, tail_steps, whole_steps
+from paged_cases import (DEV, attention_case as _attention_case, pages as _pages, rnd, run_logged,
+                         step_context as _step_context)
 from tiny import random_tokens
 
 pytestmark = pytest.mark.gpu
-DEV = torch.device("cuda:0")
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 # bfloat16 logits against the 64-bit plain implementation, as fractions of the logits' standard
@@ -30,42 +31,6 @@ SHARP = 3.0        # where the queries are scaled up so that single keys decide,
 # plain implementation taking the run's own choices (`routes=`), and the choices themselves must be the
 # plain router's wherever its margin is at least this.  The 32-bit comparison forces nothing.
 CLOSE_CALL = 0.02
-
-
-def rnd(*shape, seed=0, scale=1.0):
-    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
-
-
-def run_logged(engine, steps, routed_layers):
-    """`replays.run_steps` with the routed layers' choices: ({(request, position): logits row},
-    {request: {layer: [position] -> chosen experts}}).  Every step asks for all of its positions."""
-    slots, pos, rows, routes = {}, {}, {}, {}
-    for st in steps:
-        ents = st["entries"]
-        for e in ents:
-            assert e["want"] == list(range(len(e["tokens"])))
-            if e["id"] not in slots:
-                slots[e["id"]] = engine.new_sequence()
-                pos[e["id"]] = 0
-        ctx = engine.build_context([slots[e["id"]] for e in ents], [e["tokens"] for e in ents], [e["want"] for e in ents])
-        log = ctx._memo["route_log"] = []
-        logits = engine.model.forward(ctx).cpu().numpy()
-        engine.cache.commit(ctx.new_lengths)
-        assert len(log) == len(routed_layers)
-        chosen = [c.cpu().numpy() for c in log]
-        r = 0
-        for e in ents:
-            for w in e["want"]:
-                rows[(e["id"], pos[e["id"]] + w)] = logits[r]
-                for layer, c in zip(routed_layers, chosen):
-                    routes.setdefault(e["id"], {}).setdefault(layer, {})[pos[e["id"]] + w] = c[r]
-                r += 1
-            pos[e["id"]] += len(e["tokens"])
-        assert r == logits.shape[0]
-        for rid in st["end"]:
-            engine.end_sequence(slots.pop(rid))
-        engine.cache.check_invariants()
-    return rows, routes
 
 
 def check(engine, steps, plain, reqs, dtype, what, loosen=1.0, f32_abs=F32_ABS):
@@ -160,20 +125,6 @@ def test_lightning_scan_kernels(heads, dim, vdim, lens):
         assert (y.cpu().float() - y_want.float()).abs().max() < tol
 
 
-def _pages(lens, seed, n_pages=40):
-    """Shuffled page tables for sequences of the given lengths."""
-    rng = np.random.default_rng(seed)
-    order = rng.permutation(n_pages)
-    cols = max((l + 63) // 64 for l in lens)
-    table = torch.full((len(lens), cols), -1, dtype=torch.int32)
-    at = 0
-    for b, l in enumerate(lens):
-        for c in range((l + 63) // 64):
-            table[b, c] = int(order[at])
-            at += 1
-    return table
-
-
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H, G, D, V, taps, rot", [(6, 3, 24, 40, 4, 16), (9, 1, 8, 24, 1, 4), (2, 1, 12, 5, 3, 2),
                                                    (4, 4, 16, 16, None, 0), (2, 2, 64, 32, 6, 64)])
@@ -218,36 +169,6 @@ def test_convolution_rotation_blend_and_cache_write(dtype, H, G, D, V, taps, rot
         assert (a - b).abs().max() < (2e-5 if name in ("own values", "state") else tol), name
 
 
-def _attention_case(dtype, H, G, D, V, lens, new, window, cap, seed, needle=None):
-    """Random pages of a NaN-poisoned pool; `needle` = (sequence, key position, kv head): that key is made
-    to stand out for the sequence's last query, and its value row is large."""
-    from minfer_amd.cache.paged import v_page_shape
-    rng = np.random.default_rng(seed)
-    table = _pages(lens, seed)
-    kc = torch.full((40, G, 64, D), float("nan"), dtype=dtype)
-    vc = torch.full((40,) + v_page_shape(G, V, dtype), float("nan"), dtype=dtype)
-    for b, l in enumerate(lens):
-        for p in range(l):
-            page = int(table[b, p // 64])
-            kc[page, :, p % 64] = rnd(G, D, seed=seed * 1000 + b * 100 + p).to(dtype)
-            for g in range(G):
-                plain_ops._store_v(vc, page, p % 64, g, rnd(V, seed=seed * 777 + b * 100 + p + g))
-    n = sum(new)
-    q = rnd(n, H * D, seed=seed + 5).to(dtype)
-    pos = torch.cat([torch.arange(l - m, l) for l, m in zip(lens, new)]).to(torch.int32)
-    seq = torch.repeat_interleave(torch.arange(len(lens), dtype=torch.int32), torch.tensor(new)).to(torch.int32)
-    if needle is not None:
-        b, p, g = needle
-        page = int(table[b, p // 64])
-        row = int(np.cumsum(new)[b]) - 1
-        key = kc[page, g, p % 64].float()
-        for h in range(g * (H // G), (g + 1) * (H // G)):
-            q[row, h * D:(h + 1) * D] = (key * 6.0).to(dtype)          # q . k = 6 |k|^2 for this key
-        plain_ops._store_v(vc, page, p % 64, g, torch.full((V,), 50.0))
-    temp = torch.tensor(rng.uniform(0.7, 1.4, H), dtype=torch.float32)
-    return q, kc, vc, table, pos, seq, temp
-
-
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H, G, D, V, window, cap", [(6, 3, 24, 40, 17, 8.0), (9, 1, 8, 24, 5, 0.0), (2, 1, 12, 5, 1, 30.0),
                                                      (4, 4, 16, 16, 0, 0.0), (16, 2, 128, 64, 70, 50.0)])
@@ -285,17 +206,6 @@ def test_a_key_at_the_window_edge_decides_or_is_not_seen(dtype, window, back, in
             assert (row[2:] - 50.0).abs().max() < 0.5, (lens, new)
         else:
             assert row[2:].abs().max() < 10.0, (lens, new)
-
-
-def _step_context(lens, new, table, pos, seq):
-    from minfer_amd.engine.batch import StepContext
-    n = sum(new)
-    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
-    return StepContext(cache=None, n_tokens=n, n_seqs=len(lens), token_ids=i32([0] * n), positions=pos.to(DEV),
-                       seq_of_tok=seq.to(DEV), cu_seqlens=i32(np.concatenate([[0], np.cumsum(new)]).tolist()),
-                       start_pos=i32([l - m for l, m in zip(lens, new)]), slot_ids=i32(list(range(len(lens)))),
-                       logit_rows=None, page_tables={}, max_len=max(lens), max_new=max(new), all_decode=all(m == 1 for m in new),
-                       host_new=list(new), host_start=[l - m for l, m in zip(lens, new)])
 
 
 @pytest.mark.parametrize("H, G, D, V, window, cap", [(6, 3, 32, 48, 17, 8.0), (8, 2, 96, 48, 40, 30.0), (4, 4, 16, 16, 0, 0.0),

@@ -152,12 +152,15 @@ def test_engine_on_stand_ins_random_configuration(tmp_path, monkeypatch):
     assert _rel(run_steps(eng, chunk_steps(reqs, [list(reqs)], sizes=(2, 31, 1))), ref) < 1e-4
 
 
-def test_greedy_generation_on_stand_ins(tmp_path, monkeypatch):
-    """`generate` with its scheduler, slots and decode sessions, tokens against the plain model."""
+@pytest.mark.parametrize("name", ["B", "A"])
+def test_greedy_generation_on_stand_ins(tmp_path, monkeypatch, name):
+    """`generate` with its scheduler, slots and decode sessions, tokens against the plain model.  In "A" a
+    cache group that gives pages back comes before one that does not: the first step of a decode session
+    brings the page tables of both."""
     plain_ops.install(monkeypatch)
     from minfer_amd import Engine, generate, load_model
     from minfer_amd.sampling import SamplingParams
-    folder = write_nodutar(str(tmp_path / "gen"), ND_B, seed=8)
+    folder = write_nodutar(str(tmp_path / "gen"), ND[name], seed=8)
     plain = pn.PlainNodutar.from_folder(folder)
     eng = Engine(load_model(folder, dtype="float32", device="cpu"), max_tokens=64 * 6, max_seqs=2)
     prompts = [[5, 9, 20, 7], [11], [25, 3, 3, 3, 8, 1, 44]]
