@@ -52,7 +52,7 @@ ND_B = dict(architecture="Nodutar", vocab=97, width=64, norm=dict(eps=1e-4), lay
 # every layer passed three times; a chunk one longer than a page; one expert of two
 ND_C = dict(architecture="Nodutar", vocab=400, width=128, norm=dict(eps=1e-6), loop=dict(start=0, stop=2, times=3), layers=[
     dict(parallel(left(8, 2, 64, 64, 0.125, 65, 32), right(4, 64, 64), 1.2, 0.8), mlp=moe(4, 2, 64)),
-    dict(attention(2, 2, 64, 1.0), mlp=moe(2, 1, 100)),
+    dict(attention(2, 2, 64, 0.25), mlp=moe(2, 1, 100)),
 ])
 
 ND = {"A": ND_A, "B": ND_B, "C": ND_C}

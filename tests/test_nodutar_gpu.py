@@ -20,8 +20,10 @@ from tiny import random_tokens
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-# bfloat16 logits against the 64-bit plain implementation, as fractions of the logits' standard deviation;
-# 32-bit in absolute terms (times the logits' standard deviation where that is above one)
+# bfloat16 logits against the 64-bit plain implementation, as fractions of the logits' standard deviation, at
+# three runs of a layer and growing with the root of their number beyond (every run adds roundings of its own:
+# the engine's own composition on host stand-ins that round at the same places and compute in 64 bits in
+# between differs from the plain implementation by up to 3.4 % rms at the six runs of "A"); 32-bit in absolute terms (times the logits' standard deviation where that is above one)
 BF16_RMS, BF16_MAX, F32_ABS = 0.04, 0.2, 2e-4
 SHARP = 3.0
 # a router decides a token between two experts whose logits differ by less than this differently in bfloat16
@@ -33,6 +35,7 @@ CLOSE_CALL = 0.05
 
 def check(engine, steps, plain, reqs, dtype, what, loosen=1.0, f32_abs=F32_ABS):
     runs = plain.routed_runs()
+    loosen = loosen * max(1.0, len(pn.run_order(plain.cfg)) / 3.0) ** 0.5
     rows, routes = run_logged(engine, steps, runs)
     assert rows, "nothing was produced"
     for rid, toks in reqs.items():
