@@ -68,11 +68,12 @@ def parse():
                     help="cache size in tokens (default: batch x context, or what fits in free memory if less)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--only", choices=["decode", "prefill"], help="run one part (for profiles); prints no JSON line")
-    ap.add_argument("--design", choices=["tabezen", "lagedra"], default=None,
+    ap.add_argument("--design", choices=["tabezen", "lagedra", "nodutar"], default=None,
                     help="instead of the default workload: prefill and decode of this design at a few layer sizes "
-                         "beside the Qwen2 decoder of the same width, depth and feed-forward size, kernel by kernel")
+                         "beside its nearest relative of the same width, depth and feed-forward size (the Qwen2 "
+                         "decoder; for nodutar, Lagedra), kernel by kernel")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes to run")
-    ap.add_argument("--design-model", default=None, choices=["tabezen", "lagedra", "qwen2"],
+    ap.add_argument("--design-model", default=None, choices=["tabezen", "lagedra", "nodutar", "qwen2"],
                     help="with --design and --only: which of the two models runs the one part (for profiles; "
                          "default: the design itself)")
     return ap.parse_args()
@@ -269,6 +270,21 @@ def lagedra_config(width, layers, heads, ff, dim=128, vdim=128, window=1024, exp
                 layers=[dict(lin if (i // 2) % 2 == 0 else att, mlp=dense if i % 2 == 0 else routed) for i in range(layers)])
 
 
+def nodutar_config(width, layers, heads, ff, dim=128, vdim=128, chunk=1024, experts=8, top=2, vocab=32768):
+    """Attention with a penalty on distance and the side-by-side mixer (chunked attention beside the gated
+    recurrence) in turn, every layer with routed experts of ff / top values, `top` of them a token; head sizes,
+    kv heads, the chunk (Lagedra's window) and the recurrence's state as in `lagedra_config`."""
+    kv = max(1, heads // 4)
+    far = dict(type="attention", mixer=dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5))
+    both = dict(type="parallel", mixer=dict(
+        left=dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=dim ** -0.5, mask=dict(size=chunk),
+                  rot=dict(base=10000.0, dims=dim // 2)),
+        right=dict(heads=heads, dim=dim, vdim=vdim), left_scale=1.0, right_scale=1.0))
+    routed = dict(kind="moe", expert=dict(ff=ff // top), router=dict(experts=experts, top=top))
+    return dict(architecture="Nodutar", vocab=vocab, width=width, norm=dict(eps=1e-6),
+                layers=[dict(both if i % 2 == 0 else far, mlp=routed) for i in range(layers)])
+
+
 def qwen2_like(width, layers, heads, ff, vocab=32768):
     """The Qwen2 decoder of the same width, depth, head count and feed-forward size (head size 128)."""
     return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
@@ -282,7 +298,8 @@ DESIGN_SIZES = {
 }
 
 
-DESIGN_CONFIGS = {"tabezen": tabezen_config, "lagedra": lagedra_config, "qwen2": qwen2_like}
+DESIGN_CONFIGS = {"tabezen": tabezen_config, "lagedra": lagedra_config, "nodutar": nodutar_config, "qwen2": qwen2_like}
+NEAREST = {"tabezen": "qwen2", "lagedra": "qwen2", "nodutar": "lagedra"}      # the model a design is measured beside
 
 
 def traced_step(eng, slots, toks, want):
@@ -377,7 +394,7 @@ def run_design(a) -> int:
     for name in a.design_sizes.split(","):
         size = DESIGN_SIZES[name]
         row = {"size": size}
-        for label in (a.design, "qwen2"):
+        for label in (a.design, NEAREST[a.design]):
             print(f"{name}: {label} ...", file=sys.stderr, flush=True)
             row[label] = design_point(DESIGN_CONFIGS[label](**size), a, dtype, elem)
             if a.design == "tabezen":

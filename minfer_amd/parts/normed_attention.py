@@ -78,8 +78,9 @@ class NormedAttention(Mixer):
             s[n["q_norm"]] = TensorSpec((self.dim,), init="ones")
             s[n["k_norm"]] = TensorSpec((self.dim,), init="ones")
         if self.distance is not None:
-            s[self.distance[0]] = TensorSpec((self.nh,))
-            s[self.distance[1]] = TensorSpec((self.nh,))
+            # random weights: positive numbers, or the logarithm has no value
+            s[self.distance[0]] = TensorSpec((self.nh,), init="halves")
+            s[self.distance[1]] = TensorSpec((self.nh,), init="halves")
         return s
 
     def load(self, get):
