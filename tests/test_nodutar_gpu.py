@@ -69,7 +69,7 @@ def check(engine, steps, plain, reqs, dtype, what, loosen=1.0, f32_abs=F32_ABS):
 # ------------------------------------------------------------------ kernels alone
 @pytest.mark.parametrize("heads, dim, vdim, lens", [(3, 20, 12, (1, 5, 200, 64, 129)), (1, 40, 72, (700,)),
                                                     (2, 136, 16, (3, 128, 65)), (3, 5, 7, (1, 1, 1)), (2, 128, 130, (300, 2)),
-                                                    (6, 32, 64, (1, 1, 1, 1, 1, 1, 1)), (1, 256, 8, (66,))])
+                                                    (5, 32, 48, (1, 1, 1, 1, 1, 1, 1)), (1, 256, 8, (66,))])
 def test_gated_scan_kernels(heads, dim, vdim, lens):
     """Ragged sequences, carried state, shuffled slots; the sequential and the chunked form; the norm per head."""
     from minfer_amd.kernels import ops
@@ -103,7 +103,7 @@ def test_gated_scan_kernels(heads, dim, vdim, lens):
 @pytest.mark.parametrize("H, G, D, V, gains, rot, v_from_k, vrot", [
     (6, 3, 24, 40, True, 16, False, True), (9, 1, 10, 10, False, 0, True, False), (2, 1, 12, 6, True, 2, False, True),
     (4, 4, 16, 16, True, 16, False, False), (2, 2, 64, 32, False, 64, False, True), (3, 1, 130, 130, False, 0, True, False),
-    (8, 4, 128, 128, True, 64, False, True)])
+    (6, 2, 128, 64, True, 32, False, True)])
 def test_normed_rotated_queries_keys_values_and_the_turn_back(dtype, H, G, D, V, gains, rot, v_from_k, vrot):
     """Sequences that bring 1, 2, 70 and 5 tokens onto 0, 3, 60 and 127 held ones, into shuffled pages."""
     from minfer_amd.cache.paged import v_page_shape
@@ -151,7 +151,7 @@ def _far(H, seed):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H, G, D, V, chunk, far", [(6, 3, 24, 40, 17, False), (9, 1, 8, 24, 0, True), (2, 1, 12, 5, 1, False),
-                                                    (4, 4, 16, 16, 64, True), (16, 2, 128, 64, 70, False), (4, 1, 48, 48, 0, True),
+                                                    (4, 4, 16, 16, 64, True), (16, 2, 128, 64, 70, False), (6, 2, 48, 48, 0, True),
                                                     (3, 3, 10, 10, 100, False)])
 def test_chunks_and_distance_in_the_plain_attention_kernel(dtype, H, G, D, V, chunk, far):
     """Prompts, portions on held tokens and single tokens in one launch, over shuffled pages."""
@@ -170,8 +170,8 @@ def test_chunks_and_distance_in_the_plain_attention_kernel(dtype, H, G, D, V, ch
 
 
 @pytest.mark.parametrize("H, G, D, V, chunk, far", [(6, 3, 32, 48, 17, False), (8, 2, 96, 48, 0, True), (4, 4, 16, 16, 64, True),
-                                                    (16, 2, 128, 64, 70, False), (7, 7, 48, 16, 1, False), (4, 1, 48, 48, 0, True),
-                                                    (8, 4, 128, 128, 65, False), (2, 1, 64, 128, 100, True)])
+                                                    (16, 2, 128, 64, 70, False), (7, 7, 48, 16, 1, False), (6, 2, 48, 48, 0, True),
+                                                    (6, 2, 128, 128, 65, False), (2, 1, 64, 128, 100, True)])
 @pytest.mark.parametrize("new", [(1, 130, 3, 1, 40), (1, 64, 64, 300, 65), (1, 1, 1, 2, 17), (1, 1, 1, 1, 1)])
 def test_chunks_and_distance_in_the_matrix_core_attention_kernel(H, G, D, V, chunk, far, new):
     """Blocks of 16 tokens that lie across a chunk's edge, and a decode step whose keys split over waves."""
