@@ -1,5 +1,5 @@
 """Nodutar: a decoder whose layers put a norm before and behind each branch,
-x <- x + N1b(mixer(N1(x))), x <- x + N2b(ff(N2(x))), with norms whose weights are stored around zero; a run of
+x <- x + N1b(mixer(N1(x))), x <- x + N2b(ff(N2(x))), with RMS norms whose gain is one plus the stored weight; a run of
 consecutive layers may be passed several times with the same weights, every pass with a cache and state of its
 own and the embedding output added to the stream in front of every pass but the first.  A mixer is softmax
 attention whose values are its keys as projected, with unit-normed queries and keys and a logarithmic penalty
@@ -36,7 +36,7 @@ def _attention_sizes(raw: Any, where: str, chunked: bool) -> Dict[str, Any]:
         raise ConfigError(f"{where}: 'heads' {out['heads']} is not a multiple of 'kv_heads' {out['kv_heads']}")
     if not chunked:
         if out["vdim"] != out["dim"]:
-            raise ConfigError(f"{where}: the values are the keys, so 'vdim' {out['vdim']} must equal 'dim' {out['dim']}")
+            raise ConfigError(f"{where}: the keys serve as values, so 'vdim' {out['vdim']} must equal 'dim' {out['dim']}")
         return out
     out["mask"] = dict(size=KeyReader(r.raw_value("mask") or {}, where + ".mask").integer("size"))
     k = KeyReader(r.raw_value("rot") or {}, where + ".rot")

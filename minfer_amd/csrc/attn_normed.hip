@@ -8,7 +8,7 @@
 //   v:    its own projection, or (`v_from_k`) the key head as projected, before the norm; with value
 //         tables [positions][V / 2] its pairs (2m, 2m + 1) turn by the token's angle m, and it is
 //         cached so;
-//   the attention's result per head is turned back by the query token's angles (`unrotate_kernel`),
+//   the attention's result per head is rotated back by the query token's angles (`unrotate_kernel`),
 //   multiplied by a scale and rounded to the run type.
 //
 // `qk_norm_prep_kernel`: a workgroup per (token, head of q, k or v): the head in LDS, the sum of squares

@@ -1,4 +1,4 @@
-// Linear attention whose forget gate, one per key channel and token, also decides what is written
+// Linear attention whose forget gate, one per key channel and token, sets the input gate as well
 // (the HGRN2 recurrence), over the ragged batch of a step, state in 32-bit per sequence slot.
 //
 // Per head, with q_t = silu(q projection) (dim values), v_t the value projection (vdim values) and

@@ -1,4 +1,4 @@
-"""Linear attention in which the forget gate also decides what is written (HGRN2): a fixed-size matrix
+"""Linear attention whose forget gate a sets the input gate as well, 1 - a (HGRN2): a fixed-size matrix
 state per sequence and head instead of keys and values.
 
 q = silu(Wq x) (heads x dim), v = Wv x (heads x v_dim), a = l + (1 - l) sigmoid(Wf x + b) per head and key

@@ -91,7 +91,7 @@ class ScalarRMSNorm(RMSNorm):
 
 @register_norm("offset_rmsnorm")
 class OffsetRMSNorm(GroupRMSNorm):
-    """RMS norm whose weight is stored around zero: x / sqrt(mean(x^2) + eps) * (1 + w).  The gain 1 + w is
+    """RMS norm whose gain is one plus the stored weight: x / sqrt(mean(x^2) + eps) * (1 + w).  The gain 1 + w is
     formed once, in 32-bit, when the weights arrive, so every kernel and fold of the plain norm serves it,
     also the one that adds a normed branch result into the stream.  params: size, eps, weight (tensor name)."""
 

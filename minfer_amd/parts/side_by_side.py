@@ -1,4 +1,4 @@
-"""Two mixers side by side off the same input, their results scaled and summed:
+"""Two mixers on one input, their results scaled and summed:
 y = left_scale left(x) + right_scale right(x).
 
 Either side is any registered mixer that takes an `out_scale` (applied to its result before its last

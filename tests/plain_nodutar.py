@@ -6,9 +6,9 @@ N(x) = x / sqrt(mean(x^2) + eps) (1 + w); a run of consecutive layers may be pas
 the same weights (every pass with a cache and state of its own), the embedding output being added to
 the stream in front of every pass but the first.  A mixer is softmax attention whose values are its
 keys as projected, with unit-normed queries and keys and a logarithmic penalty on distance; or two
-mixers side by side, scaled and summed: chunked softmax attention with normed, partly rotated queries
-and keys and values that are rotated by their own position and turned back by the query's, beside a
-gated linear recurrence whose forget gate also decides what is written.  A feed-forward is a mixture
+mixers on one input, scaled and summed: chunked softmax attention with normed, partly rotated queries
+and keys and values that are rotated by their own position and rotated back by the query's, beside a
+gated linear recurrence whose input gate is one minus its forget gate.  A feed-forward is a mixture
 of silu-gated experts; the router's weights are the softmax over the chosen logits.  The head is the
 embedding table.
 """
@@ -62,7 +62,7 @@ def unit_rms(x, eps: float):
 
 
 def offset_norm(x, w, eps: float):
-    """The design's norm: the weight is stored around zero."""
+    """The design's norm: the gain is one plus the stored weight."""
     return unit_rms(x, eps) * (1.0 + w)
 
 
@@ -148,7 +148,7 @@ def distance_attention(h, w, prefix: str, m, eps: float):
 def chunked_rotary_attention(h, w, prefix: str, m, eps: float):
     """Softmax attention inside chunks of mask.size positions counted from 0, over one whole sequence:
     normed (weighted) queries and keys, rotation in pairs over the first rot.dims values, values rotated
-    by their own position over all their pairs and the head's sum turned back by the query's."""
+    by their own position over all their pairs and the head's sum rotated back by the query's."""
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     base, dims, size = m["rot"]["base"], m["rot"]["dims"], m["mask"]["size"]

@@ -134,7 +134,7 @@ def test_normed_rotated_queries_keys_values_and_the_turn_back(dtype, H, G, D, V,
         (plain_ops.unrotate if side == "plain" else ops.unrotate)(o, mv(vt), mv(pos), H, 1.3)
         outs.append([t.cpu().float() for t in (q, kc, vc, o)])
     tol = 3e-5 if dtype == torch.float32 else 1e-2          # bfloat16: a rounding apart, relative to the value
-    for name, a, b in zip(("q", "k pages", "v pages", "turned back"), *outs):
+    for name, a, b in zip(("q", "k pages", "v pages", "rotated back"), *outs):
         assert ((a - b).abs() / b.abs().clamp(min=1.0)).max() < tol, name
     if vt is not None and dtype == torch.float32:        # turning back undoes the turn
         x = (rnd(n, H * V, seed=12)).to(DEV)
