@@ -6,8 +6,8 @@
 //         given; then values 2i and 2i + 1, i < rot / 2, turn by the token's angle i (tables
 //         [positions][rot / 2]); the values from `rot` on pass;
 //   v:    its own projection, or (`v_from_k`) the key head as projected, before the norm; with value
-//         tables [positions][V / 2] its pairs (2m, 2m + 1) turn by the token's angle m, and it is
-//         cached so;
+//         tables [positions][V / 2] its pairs (2m, 2m + 1) turn by the token's angle m on the way into the
+//         cache;
 //   the attention's result per head is rotated back by the query token's angles (`unrotate_kernel`),
 //   multiplied by a scale and rounded to the run type.
 //

@@ -4,9 +4,9 @@ else a design asks of its attention, each a parameter:
 q = Wq x, k = Wk x (no biases); every q and k head over its root mean square (eps inside the root), times a
 gain vector shared by the heads where the design has one -> the rotation in neighbouring pairs over the first
 values of a head, where it has one -> values: v = Wv x, or the key heads as projected, before their norm
-(`values_from_keys`: there is no Wv then) -> with `value_rotation`, the value of position j is turned by j over
-all its pairs (a position encoding of its own, whatever the keys have) and cached so, and every head's result
-at position i is rotated back by i -> query head h reads kv head h // (heads / kv_heads); mask: all earlier
+(`values_from_keys`: there is no Wv then) -> with `value_rotation`, a value row goes into the cache rotated by
+its own position over all its pairs (an encoding of the values' own, independent of the keys' rotation), and a
+head's weighted sum for the query at position i is rotated by -i -> query head h reads kv head h // (heads / kv_heads); mask: all earlier
 positions, the last `window` of them, or (`chunk`) those of the token's own chunk of that many positions
 counted from 0 -> s = q . k scale, less a penalty on distance a[h] ln(1 + b[h] (i - j)) where the design has
 one -> ordinary softmax, o = sum p_j v_j, times `out_scale` -> Wo.
