@@ -56,6 +56,7 @@ class KVRequest:
     window: Optional[int] = None      # None: all earlier positions
     v_head_dim: Optional[int] = None  # width of a value row where it is not that of a key row
     chunk: Optional[int] = None       # a position reads only its own chunk of this many positions, counted from 0
+    keep_first: Optional[int] = None  # with a window: the first so many positions stay in sight of every later one
 
     @property
     def value_dim(self) -> int:
@@ -170,8 +171,9 @@ class KVGroup:
     def drop_left_of_window(self, slot: int, length: int) -> None:
         first = self.first_needed_page(length)
         row = self.pages[slot]
-        gone = [p for p in row[:first] if p >= 0]
-        for i in range(min(first, len(row))):
+        kept = ((self.request.keep_first or 0) + PAGE - 1) // PAGE      # the pages of the positions that stay in sight
+        gone = [p for p in row[kept:first] if p >= 0]
+        for i in range(kept, min(first, len(row))):
             row[i] = -1
         self._give(gone)
 

@@ -10,7 +10,10 @@
 //   s_j = cap tanh((q . k_j) scale temp[h] / cap), keys j with 0 <= p - j < window, ordinary softmax,
 //   o = sum_j p_j v_j.
 // The attention kernels also take a mask in chunks (a token sees the keys of its own chunk of `chunk`
-// positions counted from 0, up to itself) and a penalty on distance, s_j -= a[h] ln(1 + b[h] (p - j)).
+// positions counted from 0, up to itself), a penalty on distance, s_j -= a[h] ln(1 + b[h] (p - j)), a number per
+// head and distance that joins the score, s_j += bias[h][min(p - j, n_bias - 1)] (a table the host lays out by
+// distance, whatever rule groups the distances), and, with a window, the sequence's first `keep_first`
+// positions, which every later token goes on seeing (split 0 walks them before its own keys).
 //
 // `qkv_conv_prep_kernel`: one workgroup per (token, head of q, k or v); convolution of the head's channels
 // into LDS, then rotation, blending, the cache write and q rounded to the run type.
@@ -125,7 +128,8 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
     int pt_stride, const int* __restrict__ positions, const int* __restrict__ seq_of_tok,
     const float* __restrict__ temp, T* __restrict__ out, float* __restrict__ part, int nh, int nk, int D, int V,
     int VP, float scale, float cap, int window, int chunk, const float* __restrict__ far_a,
-    const float* __restrict__ far_b, int n_splits, int split_len) {
+    const float* __restrict__ far_b, int keep_first, const float* __restrict__ bias, int n_bias, int n_splits,
+    int split_len) {
   extern __shared__ float lds[];
   float* sq = lds;                              // [GC][D]
   float* sc = sq + MF_CAP_GC * D;               // [GC][KEYS]
@@ -147,8 +151,8 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
   int lo = window > 0 ? max(0, p - window + 1) : 0;
   if (chunk > 0) lo = max(lo, p / chunk * chunk);
   // a windowed token's splits start at its window's first key, so that all of them have keys
-  const int j_begin = lo + split * split_len;
-  const int j_end = min(p + 1, j_begin + split_len);
+  const int main_begin = lo + split * split_len;
+  const int main_end = min(p + 1, main_begin + split_len);
 
   for (int i = threadIdx.x; i < gcount * D; i += 256)
     sq[i] = to_f32(q[((size_t)t * nh + h0) * D + i]);
@@ -169,7 +173,10 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
   const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
   __syncthreads();
 
-  // rounds of 256 keys from the half page of the first key on: a round's 32-key groups are half pages
+  // rounds of 256 keys from the half page of the first key on: a round's 32-key groups are half pages.  The walk
+  // runs once over the sequence's kept first keys, where they lie before the window (split 0), and once over the
+  // split's own keys; both calls are uniform over the workgroup.
+  auto walk = [&](const int j_begin, const int j_end) {
   for (int cb = j_begin < j_end ? (j_begin & ~31) : j_end; cb < j_end; cb += MF_CAP_KEYS) {       // (a split may be empty)
     // phase 1: the scores of key cb + thread (-inf outside the token's keys)
     {
@@ -205,6 +212,7 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
         float x = s[g] * tm[g];
         if (cap > 0.f) x = cap * tanhf(x * inv_cap);
         if (far_a && valid) x -= fa[g] * log1pf(fb[g] * (float)(p - j));
+        if (bias && valid && g < gcount) x += bias[(size_t)(h0 + g) * n_bias + min(p - j, n_bias - 1)];
         sc[g * MF_CAP_KEYS + threadIdx.x] = valid ? x : -INFINITY;
       }
     }
@@ -270,6 +278,9 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
     }
     __syncthreads();
   }
+  };
+  if (keep_first > 0 && split == 0 && lo > 0) walk(0, min(keep_first, lo));
+  walk(main_begin, main_end);
 
   // add the key residues, in their order
 #pragma unroll
@@ -345,11 +356,12 @@ MF_API int mf_qkv_conv_prep(const float* qkv, const float* conv_w, int taps, flo
 MF_API int mf_capped_attn(const void* q, const void* kc, const void* vc, const int* page_table, int pt_stride,
                           const int* positions, const int* seq_of_tok, const float* temp, void* out, float* part,
                           int is_bf16, int n_tok, int nh, int nk, int D, int V, float scale, float cap, int window,
-                          int chunk, const float* far_a, const float* far_b, int n_splits, int split_len,
-                          hipStream_t stream) {
+                          int chunk, const float* far_a, const float* far_b, int keep_first, const float* bias,
+                          int n_bias, int n_splits, int split_len, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (nk <= 0 || nh % nk || D <= 0 || D > 512 || V <= 0 || V > 256 || n_splits < 1 || n_splits > 64 ||
-      split_len < 1 || (n_splits > 1 && !part) || !temp || chunk < 0 || (far_a != nullptr) != (far_b != nullptr))
+      split_len < 1 || (n_splits > 1 && !part) || !temp || chunk < 0 || (far_a != nullptr) != (far_b != nullptr) ||
+      keep_first < 0 || (keep_first > 0 && chunk > 0) || (bias && n_bias < 1))
     return (int)hipErrorInvalidValue;
   int VP = 1;
   while (VP < V) VP *= 2;
@@ -360,7 +372,7 @@ MF_API int mf_capped_attn(const void* q, const void* kc, const void* vc, const i
   if (is_bf16) {
     capped_attn_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table,
                                                          pt_stride, positions, seq_of_tok, temp, (bf16*)out, part, nh, nk,
-                                                         D, V, VP, scale, cap, window, chunk, far_a, far_b, n_splits,
+                                                         D, V, VP, scale, cap, window, chunk, far_a, far_b, keep_first, bias, n_bias, n_splits,
                                                          split_len);
     rc = mf_launch_status();
     if (rc == 0 && n_splits > 1) {
@@ -370,7 +382,7 @@ MF_API int mf_capped_attn(const void* q, const void* kc, const void* vc, const i
   } else {
     capped_attn_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)kc, (const float*)vc, page_table,
                                                           pt_stride, positions, seq_of_tok, temp, (float*)out, part, nh,
-                                                          nk, D, V, VP, scale, cap, window, chunk, far_a, far_b, n_splits,
+                                                          nk, D, V, VP, scale, cap, window, chunk, far_a, far_b, keep_first, bias, n_bias, n_splits,
                                                          split_len);
     rc = mf_launch_status();
     if (rc == 0 && n_splits > 1) {

@@ -3,7 +3,9 @@
 // compile time: the library is built for a model's sizes).  Semantics as `capped_attn_kernel`:
 // s = cap tanh(q . k scale temp[h] / cap), keys j with 0 <= p - j < window, softmax, o = sum p_j v_j; with
 // `chunk`, a token sees the keys of its own chunk of that many positions only; with `far_a`, `far_b`,
-// s -= far_a[h] ln(1 + far_b[h] (p - j)).
+// s -= far_a[h] ln(1 + far_b[h] (p - j)); with `bias`, s += bias[h][min(p - j, n_bias - 1)]; with a window and
+// `keep_first`, every token also sees the sequence's first `keep_first` keys: the wave of split 0 walks their
+// half pages first and then jumps to the half page of its window's first key.
 //
 // A wave (a workgroup of its own) owns 16 consecutive new tokens of one sequence times RB query heads of one kv
 // head and walks the tokens' keys 32 at a time (half a page), with no LDS and no barrier; the key rows of a
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     const int* __restrict__ start_pos, const int* __restrict__ tile_seq, const int* __restrict__ tile_q0, int n_tiles,
     const float* __restrict__ temp, bf16* __restrict__ out, float* __restrict__ part, int n_splits, int split_len,
     int nh, int nk, float scale, float cap, int window, int chunk, const float* __restrict__ far_a,
-    const float* __restrict__ far_b) {
+    const float* __restrict__ far_b, int keep_first, const float* __restrict__ bias, int n_bias) {
   const int lane = threadIdx.x & 63;
   const int tile = blockIdx.x;                    // a workgroup is one wave: the waves drift apart freely
   if (tile >= n_tiles) return;
@@ -78,6 +80,10 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
   const int split = blockIdx.z;
   const int k_first = (lo & ~31) + split * split_len;
   const int k_stop = n_splits > 1 ? min(p_last + 1, k_first + split_len) : p_last + 1;
+  // the kept first keys, in half pages [0, kept_stop), where they lie before the first half page of the window;
+  // the keys between them and the window are seen by none of the tile's tokens
+  const int kept_stop = (keep_first > 0 && split == 0) ? min((keep_first + 31) & ~31, k_first) : 0;
+  auto next_step = [&](int kb) { return (kb < kept_stop && kb + 32 >= kept_stop) ? k_first : kb + 32; };
 
   // Q fragments: token `col`, values 32 ks + 8 g .. + 8 of head h0 + r
   bf16x8 qf[RB][DKS];
@@ -126,8 +132,9 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
         kn[a][ks] = v;
       }
   };
-  if (k_first < k_stop) ask_k(k_first);
-  for (int kb = k_first; kb < k_stop; kb += 32) {
+  const int kb_first = kept_stop > 0 ? 0 : k_first;
+  if (kb_first < k_stop) ask_k(kb_first);
+  for (int kb = kb_first; kb < k_stop; kb = next_step(kb)) {
     const int page = pt[kb / MF_PAGE];
     const int in_page = kb % MF_PAGE;              // 0 or 32
     bf16x8 kf[2][DKS];
@@ -135,7 +142,7 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int ks = 0; ks < DKS; ++ks) kf[a][ks] = kn[a][ks];
-    if (kb + 32 < k_stop) ask_k(kb + 32);
+    if (next_step(kb) < k_stop) ask_k(next_step(kb));
     // V^T fragments: value row 16 c + col, keys 4 g .. + 4 and 16 + 4 g .. + 4 of this half page, asked for
     // before the scores are formed
     const bf16* vbase = vc + ((((size_t)page * nk + hk) * 2 + in_page / 32) * V + col) * 32 + 4 * g;
@@ -148,11 +155,13 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     // which of this lane's 8 keys its token sees: slot j < 4: key kb + 4 g + j, else kb + 16 + 4 g + j - 4
     bool seen[8];
     float dist[8];
+    int far_row[8];      // the distance's place in a head's row of the bias table
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int key = kb + (j < 4 ? 4 * g + j : 16 + 4 * g + j - 4);
-      seen[j] = row_ok && key <= p_mine && (window <= 0 || p_mine - key < window) && key >= chunk_lo;
+      seen[j] = row_ok && key <= p_mine && (window <= 0 || p_mine - key < window || key < keep_first) && key >= chunk_lo;
       dist[j] = (float)max(0, p_mine - key);
+      far_row[j] = min(max(0, p_mine - key), n_bias - 1);
     }
     bf16x8 pf[RB];
 #pragma unroll
@@ -170,6 +179,7 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
         float y = (j < 4 ? s0[j] : s1[j - 4]) * sc[r];
         if (cap > 0.f) y = cap * fast_tanh(y * inv_cap);
         if (far_a) y -= fa[r] * __logf(1.0f + fb[r] * dist[j]);
+        if (bias) y += bias[(size_t)(h0 + r) * n_bias + far_row[j]];
         x[j] = seen[j] ? y : -INFINITY;
         mx = fmaxf(mx, x[j]);
       }
@@ -255,12 +265,13 @@ MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const i
                           const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0,
                           int n_tiles, const float* temp, void* out, float* part, int n_splits, int split_len, int n_tok,
                           int nh, int nk, int d, int v, float scale, float cap, int window, int chunk, const float* far_a,
-                          const float* far_b, hipStream_t stream) {
+                          const float* far_b, int keep_first, const float* bias, int n_bias, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (d != D || v != V || nk <= 0 || nh % nk || !temp || n_splits < 1 || n_splits > 64 ||
       (n_splits > 1 && (!part || split_len < 32 || split_len % 32)) || chunk < 0 ||
-      (far_a != nullptr) != (far_b != nullptr))
+      (far_a != nullptr) != (far_b != nullptr) || keep_first < 0 || (keep_first > 0 && chunk > 0) || (bias && n_bias < 1))
     return (int)hipErrorInvalidValue;
+  if (!bias) n_bias = 1;
   const int G = nh / nk;
   // heads of a kv head a wave takes together: four where that still leaves waves for all SIMDs
   int rb = G % 2 == 0 ? 2 : 1;
@@ -269,7 +280,8 @@ MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const i
 #define MF_GO(RB)                                                                                                          \
   capped_mfma_kernel<RB><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, \
                                                    cu_seqlens, start_pos, tile_seq, tile_q0, n_tiles, temp, (bf16*)out, part, \
-                                                   n_splits, split_len, nh, nk, scale, cap, window, chunk, far_a, far_b)
+                                                   n_splits, split_len, nh, nk, scale, cap, window, chunk, far_a, far_b, \
+                                                   keep_first, bias, n_bias)
   if (rb == 4) MF_GO(4);
   else if (rb == 2) MF_GO(2);
   else MF_GO(1);

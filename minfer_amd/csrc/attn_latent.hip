@@ -20,11 +20,15 @@
 #include "common.h"
 
 // ------------------------------------------------------------------ preparation
-// proj: 32-bit rows [q: H (DN + DR) | dkv: R + DR | gate: H] at the given offsets of a row of
-// `ld` floats.  Two blocks per token: one for the cached row, one for the queries and gates.
+// proj: 32-bit rows [dkv: R + DR | gate: H gate_w] at the given offsets of a row of `ld` floats; the queries
+// [H (DN + DR)] are rows of `ldq` floats of `q_rows` (the same buffer where one product made them all, or the
+// result of a product of their own where the queries pass a latent first).  gate_w: 1 where a head has one gate,
+// the width of a head's values where every value has its own.  Two blocks per token: one for the cached row,
+// one for the queries and gates.
 template <typename OT>
 __global__ __launch_bounds__(256) void latent_prep_kernel(
-    const float* __restrict__ proj, int ld, int off_dkv, int off_gate, const float* __restrict__ cw, float eps,
+    const float* __restrict__ proj, int ld, int off_dkv, int off_gate, int gate_w, const float* __restrict__ q_rows,
+    int ldq, const float* __restrict__ cw, float eps,
     const float* __restrict__ cs, const float* __restrict__ sn, int rd, const int* __restrict__ positions,
     const int* __restrict__ seq_of_tok, const int* __restrict__ page_table, int pt_stride, OT* __restrict__ cache,
     OT* __restrict__ q_plain, OT* __restrict__ q_abs, float* __restrict__ gate, int H, int DN, int DR, int R,
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
   const int DQ = DN + DR;
   for (int i = threadIdx.x; i < H * DQ; i += 256) {
     const int h = i / DQ, e = i % DQ;
-    const float* qh = row + (size_t)h * DQ;
+    const float* qh = q_rows + (size_t)t * ldq + (size_t)h * DQ;
     if (e < DN) {
       q_plain[((size_t)t * H + h) * DN + e] = from_f32<OT>(qh[e]);
     } else {
@@ -81,22 +85,27 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
       q_abs[((size_t)t * H + h) * DK + R + j] = from_f32<OT>(v);
     }
   }
-  for (int h = threadIdx.x; h < H; h += 256) gate[(size_t)t * H + h] = 1.0f / (1.0f + expf(-row[off_gate + h]));
+  if (gate)
+    for (int i = threadIdx.x; i < H * gate_w; i += 256)
+      gate[(size_t)t * H * gate_w + i] = 1.0f / (1.0f + expf(-row[off_gate + i]));
 }
 
-MF_API int mf_latent_prep(const float* proj, int ld, int off_dkv, int off_gate, const float* cw, float eps,
+MF_API int mf_latent_prep(const float* proj, int ld, int off_dkv, int off_gate, int gate_w, const float* q_rows,
+                          int ldq, const float* cw, float eps,
                           const float* cs, const float* sn, int rd, const int* positions, const int* seq_of_tok,
                           const int* page_table, int pt_stride, void* cache, void* q_plain, void* q_abs,
                           float* gate, int is_bf16, int n_tok, int H, int DN, int DR, int R, int write_cache,
                           hipStream_t stream) {
   if (n_tok <= 0) return 0;
-  if (rd < 0 || rd > DR || (rd & 1) || H < 1 || DN < 1 || R < 1) return (int)hipErrorInvalidValue;
+  if (rd < 0 || rd > DR || (rd & 1) || H < 1 || DN < 1 || R < 1 || gate_w < 1 || !q_rows) return (int)hipErrorInvalidValue;
   if (is_bf16)
-    latent_prep_kernel<bf16><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, cw, eps, cs, sn, rd, positions,
+    latent_prep_kernel<bf16><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, gate_w, q_rows, ldq, cw, eps, cs, sn, rd,
+                                                         positions,
                                                          seq_of_tok, page_table, pt_stride, (bf16*)cache,
                                                          (bf16*)q_plain, (bf16*)q_abs, gate, H, DN, DR, R, write_cache);
   else
-    latent_prep_kernel<float><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, cw, eps, cs, sn, rd, positions,
+    latent_prep_kernel<float><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, gate_w, q_rows, ldq, cw, eps, cs, sn, rd,
+                                                         positions,
                                                           seq_of_tok, page_table, pt_stride, (float*)cache,
                                                           (float*)q_plain, (float*)q_abs, gate, H, DN, DR, R,
                                                           write_cache);
@@ -113,7 +122,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restrict__ in, int in_stride,
                                                               const T* __restrict__ wt, T* __restrict__ out,
                                                               int out_stride, const float* __restrict__ gate,
-                                                              int n_tok, int H, int NI, int NO) {
+                                                              int gate_w, int n_tok, int H, int NI, int NO) {
   extern __shared__ float xs[];          // [TT][NI]
   const int h = blockIdx.y;
   const int t0 = blockIdx.x * MF_HW_TT;
@@ -136,25 +145,25 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restric
 #pragma unroll
     for (int tt = 0; tt < MF_HW_TT; ++tt)
       if (tt < nt) {
-        const float g = gate ? gate[(size_t)(t0 + tt) * H + h] : 1.0f;
+        const float g = gate ? gate[((size_t)(t0 + tt) * H + h) * gate_w + (gate_w > 1 ? o : 0)] : 1.0f;
         out[((size_t)(t0 + tt) * H + h) * out_stride + o] = from_f32<T>(acc[tt] * g);
       }
   }
 }
 
 MF_API int mf_headwise_linear(const void* in, int in_stride, const void* wt, void* out, int out_stride,
-                              const float* gate, int is_bf16, int n_tok, int H, int NI, int NO,
+                              const float* gate, int gate_w, int is_bf16, int n_tok, int H, int NI, int NO,
                               hipStream_t stream) {
   if (n_tok <= 0) return 0;
   const size_t lds = (size_t)MF_HW_TT * NI * sizeof(float);
-  if (H < 1 || NI < 1 || NO < 1 || lds > 64 * 1024) return (int)hipErrorInvalidValue;
+  if (H < 1 || NI < 1 || NO < 1 || lds > 64 * 1024 || (gate && gate_w != 1 && gate_w != NO)) return (int)hipErrorInvalidValue;
   dim3 grid((n_tok + MF_HW_TT - 1) / MF_HW_TT, H, (NO + 255) / 256);
   if (is_bf16)
     headwise_linear_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)in, in_stride, (const bf16*)wt, (bf16*)out,
-                                                              out_stride, gate, n_tok, H, NI, NO);
+                                                              out_stride, gate, gate_w, n_tok, H, NI, NO);
   else
     headwise_linear_kernel<float><<<grid, 256, lds, stream>>>((const float*)in, in_stride, (const float*)wt,
-                                                               (float*)out, out_stride, gate, n_tok, H, NI, NO);
+                                                               (float*)out, out_stride, gate, gate_w, n_tok, H, NI, NO);
   return mf_launch_status();
 }
 
@@ -170,8 +179,8 @@ typedef unsigned int hw_u32x4 __attribute__((ext_vector_type(4)));
 template <int MT>
 __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restrict__ in, int in_stride,
                                                             const bf16* __restrict__ wo, bf16* __restrict__ out,
-                                                            int out_stride, const float* __restrict__ gate, int n_tok,
-                                                            int H, int NI, int NO, int n_ttiles, int n_otiles) {
+                                                            int out_stride, const float* __restrict__ gate, int gate_w,
+                                                            int n_tok, int H, int NI, int NO, int n_ttiles, int n_otiles) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int task = blockIdx.x * 4 + wv;
   if (task >= H * n_otiles * n_ttiles) return;
@@ -206,7 +215,8 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
     }
   }
   if (!tok_ok) return;
-  const float g = gate ? gate[(size_t)t * H + h] : 1.0f;
+  const float* grow = gate ? gate + ((size_t)t * H + h) * gate_w : nullptr;
+  const float g = (gate && gate_w == 1) ? grow[0] : 1.0f;
   bf16* orow = out + ((size_t)t * H + h) * out_stride;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -214,12 +224,12 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
     if (o0 + 3 < NO && (out_stride & 3) == 0) {
       bf16x4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[mt][i] * g);
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[mt][i] * (gate_w > 1 ? grow[o0 + i] : g));
       *reinterpret_cast<bf16x4*>(orow + o0) = v;
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[mt][i] * g);
+        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[mt][i] * (gate_w > 1 ? grow[o0 + i] : g));
     }
   }
 }
@@ -232,8 +242,8 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
 #define MF_HW_KS_MAX 16
 __global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restrict__ in, int in_stride,
                                                            const bf16* __restrict__ wo, bf16* __restrict__ out,
-                                                           int out_stride, const float* __restrict__ gate, int n_tok,
-                                                           int H, int NI, int NO) {
+                                                           int out_stride, const float* __restrict__ gate, int gate_w,
+                                                           int n_tok, int H, int NI, int NO) {
   extern __shared__ __attribute__((aligned(16))) unsigned char hw_smem[];
   bf16* Ws = reinterpret_cast<bf16*>(hw_smem);
   const int WSTR = NI + 8;
@@ -261,7 +271,8 @@ __global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restric
     if (ks < nks && tok_ok && i < NI) xb[ks] = *reinterpret_cast<const hw_u32x4*>(xrow + i);
   }
   if (blockIdx.x * 128 + wv * 16 >= n_tok) return;      // (after the barrier; uniform over the wave)
-  const float g = (gate && tok_ok) ? gate[(size_t)t * H + h] : 1.0f;
+  const float* grow = (gate && tok_ok) ? gate + ((size_t)t * H + h) * gate_w : nullptr;
+  const float g = (grow && gate_w == 1) ? grow[0] : 1.0f;
   bf16* orow = out + ((size_t)(tok_ok ? t : 0) * H + h) * out_stride;
   for (int mt = 0; mt < NO16 / 16; ++mt) {
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -280,21 +291,21 @@ __global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restric
     if (o0 + 3 < NO && (out_stride & 3) == 0) {
       bf16x4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[i] * g);
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[i] * (gate_w > 1 ? grow[o0 + i] : g));
       *reinterpret_cast<bf16x4*>(orow + o0) = v;
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[i] * g);
+        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[i] * (gate_w > 1 ? grow[o0 + i] : g));
     }
   }
 }
 
 MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void* out, int out_stride,
-                            const float* gate, int n_tok, int H, int NI, int NO, hipStream_t stream) {
+                            const float* gate, int gate_w, int n_tok, int H, int NI, int NO, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (H < 1 || NI < 1 || NO < 1 || NI % 8 || in_stride % 8 || (uintptr_t)in % 16 || (uintptr_t)wo % 16 ||
-      (uintptr_t)out % 8)
+      (uintptr_t)out % 8 || (gate && gate_w != 1 && gate_w != NO))
     return (int)hipErrorInvalidValue;
   const int n_ttiles = (n_tok + 15) / 16;
   const size_t lds = (size_t)((NO + 15) / 16 * 16) * (NI + 8) * 2;
@@ -307,19 +318,19 @@ MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void*
       raised = true;
     }
     headwise_lds_kernel<<<dim3((n_tok + 127) / 128, H), 512, lds, stream>>>(
-        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, n_tok, H, NI, NO);
+        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO);
     return mf_launch_status();
   }
   if (n_tok <= 16) {
     const int n_otiles = (NO + 15) / 16;
     const long long tasks = (long long)H * n_otiles * n_ttiles;
     headwise_mfma_kernel<1><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(
-        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, n_tok, H, NI, NO, n_ttiles, n_otiles);
+        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO, n_ttiles, n_otiles);
   } else {
     const int n_otiles = (NO + 63) / 64;
     const long long tasks = (long long)H * n_otiles * n_ttiles;
     headwise_mfma_kernel<4><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(
-        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, n_tok, H, NI, NO, n_ttiles, n_otiles);
+        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO, n_ttiles, n_otiles);
   }
   return mf_launch_status();
 }

@@ -2,9 +2,12 @@
 // head, whose rotation turns neighbouring pairs, and whose values may be the keys as projected and may
 // be rotated themselves; and the turn back of the attention's result.
 //
-//   q, k (per head): x / sqrt(mean(x^2) + eps), times a gain vector shared by the heads where one is
-//         given; then values 2i and 2i + 1, i < rot / 2, turn by the token's angle i (tables
-//         [positions][rot / 2]); the values from `rot` on pass;
+//   q, k (per head): x / sqrt(mean(x^2) + eps) (or no norm at all), times a gain vector shared by the heads
+//         where one is given; then values 2i and 2i + 1, i < rot / 2, turn by the token's angle i (tables
+//         [positions][rot / 2]), or, in the half-split layout, value i turns with value i + rot / 2; the
+//         values from `rot` on pass.  A design that norms behind the rotation, without gains, gets the same
+//         numbers: a rotation leaves a head's sum of squares as it is, and a common factor passes through it;
+//   a layer that reads another layer's keys and values (`q_only`) has query heads only;
 //   v:    its own projection, or (`v_from_k`) the key head as projected, before the norm; with value
 //         tables [positions][V / 2] its pairs (2m, 2m + 1) turn by the token's angle m on the way into the
 //         cache;
@@ -20,8 +23,8 @@ template <typename T>
 __global__ __launch_bounds__(128) void qk_norm_prep_kernel(
     const float* __restrict__ qkv, int C, const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     int normed, const int* __restrict__ seq_of_tok, const int* __restrict__ positions, const float* __restrict__ cos_r,
-    const float* __restrict__ sin_r, int rot, const float* __restrict__ cos_v, const float* __restrict__ sin_v,
-    int v_from_k, const int* __restrict__ page_table, int pt_stride, T* __restrict__ q_out, T* __restrict__ kc,
+    const float* __restrict__ sin_r, int rot, int halves, const float* __restrict__ cos_v,
+    const float* __restrict__ sin_v, int v_from_k, const int* __restrict__ page_table, int pt_stride, T* __restrict__ q_out, T* __restrict__ kc,
     T* __restrict__ vc, int H, int G, int D, int V, int write_cache) {
   extern __shared__ float y[];
   __shared__ float scratch[2];
@@ -68,10 +71,12 @@ __global__ __launch_bounds__(128) void qk_norm_prep_kernel(
   for (int e = threadIdx.x; e < D; e += 128) {
     float v = y[e] * inv * (gain ? gain[e] : 1.0f);
     if (e < rot) {
-      const int o = e ^ 1;
+      // the value's partner and whether the value is the pair's second: neighbours, or half a rotation apart
+      const int o = halves ? (e < half ? e + half : e - half) : (e ^ 1);
+      const bool second = halves ? e >= half : (e & 1);
+      const int i = halves ? (second ? e - half : e) : (e >> 1);
       const float w = y[o] * inv * (gain ? gain[o] : 1.0f);
-      const int i = e >> 1;
-      v = (e & 1) ? v * cs[i] + w * sn[i] : v * cs[i] - w * sn[i];
+      v = second ? v * cs[i] + w * sn[i] : v * cs[i] - w * sn[i];
     }
     if (kind == 0) q_out[((size_t)t * H + head) * D + e] = from_f32<T>(v);
     else if (write_cache) kc[(((size_t)page * G + head) * MF_PAGE + in_page) * D + e] = from_f32<T>(v);
@@ -101,23 +106,25 @@ __global__ __launch_bounds__(256) void unrotate_kernel(T* __restrict__ rows, con
 
 MF_API int mf_qk_norm_prep(const float* qkv, const float* q_gain, const float* k_gain, float eps, int normed,
                            const int* seq_of_tok, const int* positions, const float* cos_r, const float* sin_r, int rot,
-                           const float* cos_v, const float* sin_v, int v_from_k, const int* page_table, int pt_stride,
+                           int halves, int q_only, const float* cos_v, const float* sin_v, int v_from_k, const int* page_table, int pt_stride,
                            void* q_out, void* kc, void* vc, int is_bf16, int n_tok, int H, int G, int D, int V,
                            int write_cache, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (H <= 0 || G <= 0 || D <= 0 || V <= 0 || rot < 0 || rot % 2 || rot > D || (rot > 0 && (!cos_r || !sin_r)) ||
       (cos_v != nullptr) != (sin_v != nullptr) || (cos_v && V % 2) || (v_from_k && V != D) || D > 8192 || V > 8192)
     return (int)hipErrorInvalidValue;
-  const int C = H * D + G * D + (v_from_k ? 0 : G * V);
+  // with q_only the rows hold the query heads alone and only they are prepared: nothing is written to the cache
+  const int C = q_only ? H * D : H * D + G * D + (v_from_k ? 0 : G * V);
   const size_t lds = (size_t)(D > V ? D : V) * sizeof(float);
-  const dim3 grid(n_tok, H + G + (v_from_k ? 0 : G));
+  const dim3 grid(n_tok, q_only ? H : H + G + (v_from_k ? 0 : G));
+  if (q_only) write_cache = 0;
   if (is_bf16)
     qk_norm_prep_kernel<bf16><<<grid, 128, lds, stream>>>(qkv, C, q_gain, k_gain, eps, normed, seq_of_tok, positions, cos_r,
-                                                           sin_r, rot, cos_v, sin_v, v_from_k, page_table, pt_stride,
+                                                           sin_r, rot, halves, cos_v, sin_v, v_from_k, page_table, pt_stride,
                                                            (bf16*)q_out, (bf16*)kc, (bf16*)vc, H, G, D, V, write_cache);
   else
     qk_norm_prep_kernel<float><<<grid, 128, lds, stream>>>(qkv, C, q_gain, k_gain, eps, normed, seq_of_tok, positions, cos_r,
-                                                            sin_r, rot, cos_v, sin_v, v_from_k, page_table, pt_stride,
+                                                            sin_r, rot, halves, cos_v, sin_v, v_from_k, page_table, pt_stride,
                                                             (float*)q_out, (float*)kc, (float*)vc, H, G, D, V, write_cache);
   return mf_launch_status();
 }

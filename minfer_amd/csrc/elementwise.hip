@@ -70,12 +70,12 @@ template <typename OT>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x,
                                                       const int* __restrict__ row_idx,
                                                       const float* __restrict__ w,
-                                                      OT* __restrict__ out, int d, float eps) {
+                                                      OT* __restrict__ out, int d, float eps, int ld) {
   __shared__ float scratch[4];
   const int row = blockIdx.x;
-  const float* xr = x + (size_t)(row_idx ? row_idx[row] : row) * d;
+  const float* xr = x + (size_t)(row_idx ? row_idx[row] : row) * ld;      // (ld > d: the first d values of longer rows)
   OT* o = out + (size_t)row * d;
-  if (d % 4 == 0 && d <= 256 * 4 * 16) {
+  if (d % 4 == 0 && ld % 4 == 0 && d <= 256 * 4 * 16) {
     if (d <= 256 * 4 * 4) rmsnorm_row_kept<OT, 4>(xr, w, o, d, eps, scratch);
     else if (d <= 256 * 4 * 8) rmsnorm_row_kept<OT, 8>(xr, w, o, d, eps, scratch);
     else rmsnorm_row_kept<OT, 16>(xr, w, o, d, eps, scratch);
@@ -98,9 +98,21 @@ MF_API int mf_rmsnorm(const float* x, const int* row_idx, const float* w, void* 
                       int out_is_bf16, int rows, int d, float eps, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (out_is_bf16)
-    rmsnorm_kernel<bf16><<<rows, 256, 0, stream>>>(x, row_idx, w, (bf16*)out, d, eps);
+    rmsnorm_kernel<bf16><<<rows, 256, 0, stream>>>(x, row_idx, w, (bf16*)out, d, eps, d);
   else
-    rmsnorm_kernel<float><<<rows, 256, 0, stream>>>(x, row_idx, w, (float*)out, d, eps);
+    rmsnorm_kernel<float><<<rows, 256, 0, stream>>>(x, row_idx, w, (float*)out, d, eps, d);
+  return mf_launch_status();
+}
+
+// the norm over the first d values of rows of ld values
+MF_API int mf_rmsnorm_cols(const float* x, int ld, const float* w, void* out, int out_is_bf16, int rows, int d, float eps,
+                           hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (d < 1 || ld < d) return (int)hipErrorInvalidValue;
+  if (out_is_bf16)
+    rmsnorm_kernel<bf16><<<rows, 256, 0, stream>>>(x, nullptr, w, (bf16*)out, d, eps, ld);
+  else
+    rmsnorm_kernel<float><<<rows, 256, 0, stream>>>(x, nullptr, w, (float*)out, d, eps, ld);
   return mf_launch_status();
 }
 
@@ -644,6 +656,20 @@ MF_API int mf_gelu_tanh(const float* x, void* out, int out_is_bf16, size_t n, hi
     gelu_tanh_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (bf16*)out, n);
   else
     gelu_tanh_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, n);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- capped logits
+// x <- cap tanh(x / cap), in place, 32-bit.
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, float cap, float inv_cap, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] * inv_cap);
+}
+
+MF_API int mf_softcap(float* x, float cap, size_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  if (!(cap > 0.f)) return (int)hipErrorInvalidValue;
+  softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, cap, 1.0f / cap, n);
   return mf_launch_status();
 }
 

@@ -7,6 +7,9 @@
 //
 // A router may add a bias per expert to its logits.  With one group, all of it kept, the weights are the
 // softmax over the chosen logits alone (the scores' common divisor cancels).
+// Further options: the scores are sigmoid(logits) instead of the softmax; a correction per expert joins the
+// scores for the choice of groups and experts only (the weights take the scores themselves); a group's score is
+// the sum of its `group_top` best (corrected) scores instead of its best; the weights are multiplied by a scale.
 //
 // Expert: g = min(gate, limit), u = clamp(up, -limit, limit), y = g sigmoid(1.702 g) (u + 1); or, with
 // `act` 1, the plain gated form y = silu(gate) up.
@@ -18,6 +21,9 @@
 #include "common.h"
 
 #define MF_MOE_MAX_EXPERTS 1024
+
+#define MF_MOE_SCORE_SOFTMAX 0
+#define MF_MOE_SCORE_SIGMOID 1
 
 // index of the largest value among a wave's candidates; ties go to the lower index
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
@@ -54,7 +60,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x
                                                        const float* __restrict__ bias, int K,
                                                        float* __restrict__ dense, int* __restrict__ chosen,
                                                        float* __restrict__ weights, int E, int n_groups, int keep,
-                                                       int top) {
+                                                       int top, int score_kind, const float* __restrict__ correction,
+                                                       int group_top, float weight_scale) {
   __shared__ float s[MF_MOE_MAX_EXPERTS], ms[MF_MOE_MAX_EXPERTS], gs[MF_MOE_MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const XT* xr = x + (size_t)t * K;
@@ -78,53 +85,75 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x
   }
   __syncthreads();
   if (wv != 0) return;              // from here on one wave: MF_WAVE_SYNC where the block form has a barrier
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
-  sum = wave_sum(sum);
-  MF_WAVE_SYNC();
-  for (int e = lane; e < E; e += 64) {
-    s[e] = s[e] / sum;
-    if (dense) dense[(size_t)t * E + e] = 0.f;
+  if (score_kind == MF_MOE_SCORE_SIGMOID) {
+    for (int e = lane; e < E; e += 64) s[e] = 1.0f / (1.0f + expf(-s[e]));
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
+    sum = wave_sum(sum);
+    MF_WAVE_SYNC();
+    for (int e = lane; e < E; e += 64) s[e] = s[e] / sum;
   }
+  for (int e = lane; e < E; e += 64)
+    if (dense) dense[(size_t)t * E + e] = 0.f;
   MF_WAVE_SYNC();
+  // an expert is chosen by its score plus the correction (the weights take the score alone); what cannot be
+  // chosen counts as minus infinity, since corrected scores may be negative
   const int per = E / n_groups;
   for (int g = lane; g < n_groups; g += 64) {
-    float b = -1.f;
-    for (int i = 0; i < per; ++i) b = fmaxf(b, s[g * per + i]);
-    gs[g] = b;
+    // the group's `group_top` largest choice scores, summed: each pass takes the best that comes behind the last
+    // one taken in the order (larger first, lower index first)
+    float total = 0.f, last_v = INFINITY;
+    int last_i = -1;
+    for (int n = 0; n < group_top && n < per; ++n) {
+      float b = -INFINITY;
+      int bi = -1;
+      for (int i = 0; i < per; ++i) {
+        const float v = s[g * per + i] + (correction ? correction[g * per + i] : 0.f);
+        const bool behind = v < last_v || (v == last_v && i > last_i);
+        if (behind && (bi < 0 || v > b)) { b = v; bi = i; }
+      }
+      if (bi < 0) break;
+      total += b;
+      last_v = b;
+      last_i = bi;
+    }
+    gs[g] = total;
   }
-  for (int e = lane; e < E; e += 64) ms[e] = -1.f;
+  for (int e = lane; e < E; e += 64) ms[e] = -INFINITY;
   MF_WAVE_SYNC();
   for (int k = 0; k < keep; ++k) {
-    float b = -2.f;
+    float b = -INFINITY;
     int bi = 0x7fffffff;
     for (int g = lane; g < n_groups; g += 64)
       if (gs[g] > b) { b = gs[g]; bi = g; }
     wave_argmax(b, bi);
+    bi = min(bi, n_groups - 1);       // (nothing finite left: scores that are not numbers)
     MF_WAVE_SYNC();
-    if (lane == 0) gs[bi] = -3.f;
-    for (int i = lane; i < per; i += 64) ms[bi * per + i] = s[bi * per + i];
+    if (lane == 0) gs[bi] = -INFINITY;
+    for (int i = lane; i < per; i += 64) ms[bi * per + i] = s[bi * per + i] + (correction ? correction[bi * per + i] : 0.f);
     MF_WAVE_SYNC();
   }
   float wsum = 0.f;
   int mine = -1;          // lane k keeps the k-th choice (top <= 64)
   for (int k = 0; k < top; ++k) {
-    float b = -2.f;
+    float b = -INFINITY;
     int bi = 0x7fffffff;
     for (int e = lane; e < E; e += 64)
       if (ms[e] > b) { b = ms[e]; bi = e; }
     wave_argmax(b, bi);
+    bi = min(bi, E - 1);
     MF_WAVE_SYNC();
-    if (lane == 0) ms[bi] = -3.f;
+    if (lane == 0) ms[bi] = -INFINITY;
     if (lane == k) mine = bi;
     wsum += s[bi];
     MF_WAVE_SYNC();
   }
   if (lane < top) {
-    const float wgt = s[mine] / (wsum + 1e-20f);
+    const float wgt = s[mine] / (wsum + 1e-20f) * weight_scale;
     if (dense) dense[(size_t)t * E + mine] = wgt;
     chosen[(size_t)t * top + lane] = mine;
     weights[(size_t)t * top + lane] = wgt;
@@ -337,15 +366,19 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 
 // ------------------------------------------------------------------ entry points
 MF_API int mf_moe_route(const void* x, int x_is_bf16, const float* router, const float* bias, int K, float* dense, int* chosen,
-                        float* weights, int n_tok, int E, int n_groups, int keep, int top, hipStream_t stream) {
+                        float* weights, int n_tok, int E, int n_groups, int keep, int top, int score_kind,
+                        const float* correction, int group_top, float weight_scale, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (K <= 0 || E <= 0 || E > MF_MOE_MAX_EXPERTS || n_groups <= 0 || E % n_groups || keep <= 0 || keep > n_groups || top <= 0 ||
-      top > 64 || top > keep * (E / n_groups))
+      top > 64 || top > keep * (E / n_groups) || group_top < 1 ||
+      (score_kind != MF_MOE_SCORE_SOFTMAX && score_kind != MF_MOE_SCORE_SIGMOID))
     return (int)hipErrorInvalidValue;
   if (x_is_bf16)
-    moe_route_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)x, router, bias, K, dense, chosen, weights, E, n_groups, keep, top);
+    moe_route_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)x, router, bias, K, dense, chosen, weights, E, n_groups, keep, top,
+                                                      score_kind, correction, group_top, weight_scale);
   else
-    moe_route_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)x, router, bias, K, dense, chosen, weights, E, n_groups, keep, top);
+    moe_route_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)x, router, bias, K, dense, chosen, weights, E, n_groups, keep, top,
+                                                      score_kind, correction, group_top, weight_scale);
   return mf_launch_status();
 }
 

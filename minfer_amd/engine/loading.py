@@ -16,7 +16,8 @@ import torch
 from ..config.base import ConfigError, read_config_json
 from ..kernels import ops
 from ..registry import config_from_dict
-from ..weights.loader import FolderWeights
+from ..weights.loader import FolderWeights, WeightError
+from ..weights.safetensors_io import SafetensorsError, open_model_files
 from ..weights.random_init import tensor_seed
 from .model import DecoderModel
 
@@ -61,11 +62,22 @@ def generation_stop_tokens(folder: str, vocab_size: int) -> Tuple[int, ...]:
     return tuple(int(t) for t in ids)
 
 
+def tensor_shapes(folder: str) -> Dict[str, Tuple[int, ...]]:
+    """name -> shape of every tensor in the folder's file(s), from the headers alone."""
+    try:
+        return {name: tuple(f.entries[name][1]) for name, f in open_model_files(folder).items()}
+    except SafetensorsError as e:
+        raise WeightError(str(e)) from None
+
+
 def load_model(folder: str, dtype="bfloat16", device="cuda:0") -> DecoderModel:
     """config.json picks the architecture; model.safetensors gives the tensors by name.  Stop
     tokens are config.json's, joined by generation_config.json's where the folder has one."""
     device = require_gpu(device)
     config = config_from_dict(read_config_json(folder))
+    if hasattr(config, "adopt_tensor_shapes"):
+        # a design may leave a size to its tensors (the rows of a table): the configuration takes it from the file
+        config.adopt_tensor_shapes(tensor_shapes(folder))
     model = DecoderModel(config.model_spec(), run_dtype(dtype), device)
     model.config = config
     expected = model.expected_tensors()

@@ -31,6 +31,7 @@ _PROTOTYPES = {
     "elementwise": {
         "mf_embed": [_P, c_int, _P, _P, c_int, c_int, c_int, _P],
         "mf_rmsnorm": [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
+        "mf_rmsnorm_cols": [_P, c_int, _P, _P, c_int, c_int, c_int, c_float, _P],
         "mf_gather_rows": [_P, _P, _P, c_int, c_int, _P],
         "mf_swiglu": [_P, c_int, _P, c_int, c_int, c_int, _P],
         "mf_convert": [_P, c_int, _P, c_int, c_size_t, _P],
@@ -45,6 +46,7 @@ _PROTOTYPES = {
         "mf_rope_pairs_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_embed_pos": [_P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
         "mf_gelu_tanh": [_P, _P, c_int, c_size_t, _P],
+        "mf_softcap": [_P, c_float, c_size_t, _P],
         "mf_weighted_sum": [_P, c_int, c_int, _P, _P, _P, c_int, c_int, _P],
         "mf_add_rows": [_P, _P, c_size_t, _P],
     },
@@ -58,15 +60,15 @@ _PROTOTYPES = {
         "mf_qkv_conv_prep": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, c_float, _P, _P, _P, c_int, _P, _P, _P,
                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_capped_attn": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_float, c_float, c_int, c_int, _P, _P, c_int, c_int, _P],
+                           c_float, c_float, c_int, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, _P],
         "mf_rope_half_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     },
     "attn_capped_mfma": {
         "mf_capped_mfma": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_int, c_float, c_float, c_int, c_int, _P, _P, _P],
+                           c_int, c_float, c_float, c_int, c_int, _P, _P, c_int, _P, c_int, _P],
     },
     "attn_normed": {
-        "mf_qk_norm_prep": [_P, _P, _P, c_float, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, _P, _P, _P,
+        "mf_qk_norm_prep": [_P, _P, _P, c_float, c_int, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, c_int, _P, c_int, _P, _P, _P,
                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_unrotate": [_P, c_int, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
     },
@@ -77,7 +79,7 @@ _PROTOTYPES = {
         "mf_head_rmsnorm": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float, _P],
     },
     "moe": {
-        "mf_moe_route": [_P, c_int, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_moe_route": [_P, c_int, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P],
         "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P],
         "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                           _P],
@@ -91,10 +93,10 @@ _PROTOTYPES = {
         "mf_scan_chunk": [],
     },
     "attn_latent": {
-        "mf_latent_prep": [_P, c_int, c_int, c_int, _P, c_float, _P, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
-        "mf_headwise_linear": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P],
-        "mf_headwise_mfma": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_latent_prep": [_P, c_int, c_int, c_int, c_int, _P, c_int, _P, c_float, _P, _P, c_int, _P, _P, _P, c_int, _P, _P,
+                           _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_headwise_linear": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_headwise_mfma": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_latent_attn": [_P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                            c_int, c_int, _P],
     },
@@ -351,8 +353,20 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
 
 
 def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor,
-            row_idx: Optional[torch.Tensor] = None) -> None:
+            row_idx: Optional[torch.Tensor] = None, cols: Optional[int] = None) -> None:
+    """out = x / sqrt(mean(x^2) + eps) * weight, row by row (row r reads x[row_idx[r]] where given).  `cols`: the norm
+    is taken over the first `cols` values of x's longer rows (the front of a product's stacked output)."""
     _need(x, "rmsnorm.x", torch.float32)
+    if cols is not None and cols != x.shape[-1]:
+        rows = x.shape[0]
+        if row_idx is not None or not 1 <= cols < x.shape[1]:
+            raise KernelError(f"rmsnorm: the first {cols} values of rows of {x.shape[1]}, with a row list or not")
+        _need(out, "rmsnorm.out", _FLOATS, (rows, cols))
+        if weight is not None:
+            _need(weight, "rmsnorm.weight", torch.float32, (cols,))
+        _check(_fn("elementwise", "mf_rmsnorm_cols")(_ptr(x), x.shape[1], _ptr(weight), _ptr(out), _is_bf16(out), rows, cols,
+                                                      float(eps), _stream()), "rmsnorm")
+        return
     d = x.shape[-1]
     rows = out.shape[0]
     _need(out, "rmsnorm.out", _FLOATS, (rows, d))
@@ -561,6 +575,14 @@ def gelu_tanh(x: torch.Tensor, out: torch.Tensor) -> None:
     _check(_fn("elementwise", "mf_gelu_tanh")(_ptr(x), _ptr(out), _is_bf16(out), x.numel(), _stream()), "gelu_tanh")
 
 
+def softcap(x: torch.Tensor, cap: float) -> None:
+    """x <- cap tanh(x / cap), in place, 32-bit."""
+    _need(x, "softcap.x", torch.float32)
+    if not cap > 0:
+        raise KernelError(f"softcap: cap {cap} must be positive")
+    _check(_fn("elementwise", "mf_softcap")(_ptr(x), float(cap), x.numel(), _stream()), "softcap")
+
+
 def weighted_sum(buffers, weights: torch.Tensor, out: torch.Tensor, row_idx: Optional[torch.Tensor] = None,
                  n_indexed: int = 0) -> None:
     """out[r] = sum_j weights[j] buffers[j][row(j, r)], added in the order of j in 32-bit.  The first
@@ -667,15 +689,17 @@ def qk_norm_prep(qkv: torch.Tensor, q_gain: Optional[torch.Tensor], k_gain: Opti
                  normed: bool, seq_of_tok: torch.Tensor, positions: torch.Tensor, rot_tables, value_tables,
                  v_from_k: bool, page_table: torch.Tensor, q_out: torch.Tensor, kcache: torch.Tensor,
                  vcache: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, v_dim: int,
-                 write_cache: bool = True) -> None:
+                 write_cache: bool = True, halves: bool = False, q_only: bool = False) -> None:
     """From the 32-bit q|k|v rows of one product (q|k alone with `v_from_k`): with `normed`, every q and k head
     over its root mean square (eps inside the root), times `q_gain` / `k_gain` (float32 `[dim]`) where given; the
     rotation in neighbouring pairs over the first 2 x columns values of a head (`rot_tables` = (cos, sin) or
     None); the value heads (their own projection, or with `v_from_k` the key heads as projected) rotated in pairs
     over all their values (`value_tables` = (cos, sin) `[positions][v_dim / 2]` or None); k and v into the cache
-    pages at the tokens' positions and q rounded into `q_out`."""
+    pages at the tokens' positions and q rounded into `q_out`.  `halves`: the rotation turns value i with value
+    i + columns instead (the half-split layout).  `q_only`: the rows hold the query heads alone (a layer that
+    reads another layer's keys and values); nothing is written to the cache."""
     n_tok = positions.numel()
-    C = n_heads * dim + n_kv_heads * dim + (0 if v_from_k else n_kv_heads * v_dim)
+    C = n_heads * dim if q_only else n_heads * dim + n_kv_heads * dim + (0 if v_from_k else n_kv_heads * v_dim)
     _need(qkv, "qk_norm_prep.qkv", torch.float32, (n_tok, C))
     for name, g in (("q_gain", q_gain), ("k_gain", k_gain)):
         if g is not None:
@@ -704,7 +728,8 @@ def qk_norm_prep(qkv: torch.Tensor, q_gain: Optional[torch.Tensor], k_gain: Opti
     _need(positions, "qk_norm_prep.positions", torch.int32, (n_tok,))
     _check(_fn("attn_normed", "mf_qk_norm_prep")(
         _ptr(qkv), _ptr(q_gain), _ptr(k_gain), float(eps), 1 if normed else 0, _ptr(seq_of_tok), _ptr(positions),
-        _ptr(cos_r), _ptr(sin_r), rot, _ptr(cos_v), _ptr(sin_v), 1 if v_from_k else 0, _ptr(page_table),
+        _ptr(cos_r), _ptr(sin_r), rot, 1 if halves else 0, 1 if q_only else 0, _ptr(cos_v), _ptr(sin_v),
+        1 if v_from_k else 0, _ptr(page_table),
         page_table.shape[1], _ptr(q_out), _ptr(kcache), _ptr(vcache), _is_bf16(q_out), n_tok, n_heads, n_kv_heads, dim,
         v_dim, 1 if write_cache else 0, _stream()), "qk_norm_prep")
 
@@ -882,11 +907,13 @@ def _need_kv_pages(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype,
 def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
                 positions: torch.Tensor, seq_of_tok: torch.Tensor, temp: torch.Tensor, out: torch.Tensor,
                 n_heads: int, n_kv_heads: int, dim: int, v_dim: int, scale: float, cap: float, window: int,
-                max_len: int, chunk: int = 0, far=None) -> None:
+                max_len: int, chunk: int = 0, far=None, keep_first: int = 0, bias: Optional[torch.Tensor] = None) -> None:
     """Each query token attends to its sequence's cache rows lo..position with
     s = cap tanh(q . k scale temp[head] / cap) (no cap where `cap` is 0), ordinary softmax; keys of
     `dim` and values of `v_dim` values.  `chunk`: a token sees only the keys of its own chunk of that many
-    positions, counted from 0.  `far` = (a, b), float32 per head: s -= a[h] ln(1 + b[h] (position - key))."""
+    positions, counted from 0.  `far` = (a, b), float32 per head: s -= a[h] ln(1 + b[h] (position - key)).
+    `keep_first`: with a window, the sequence's first so many positions stay in sight of every later token.
+    `bias` float32 `[heads][n]`: s += bias[h][min(position - key, n - 1)]."""
     n_tok = positions.numel()
     _need(q, "capped_attn.q", _FLOATS, (n_tok, n_heads * dim))
     _need(out, "capped_attn.out", q.dtype, (n_tok, n_heads * v_dim))
@@ -901,6 +928,7 @@ def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
     if max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"capped_attn: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
     far_a, far_b = _far_pair("capped_attn", far, n_heads)
+    keep_first, n_bias = _kept_and_bias("capped_attn", keep_first, window, chunk, bias, n_heads)
     # keys split over workgroups where tokens x kv heads alone do not fill the chip: at least 256 keys a split;
     # a windowed token's splits start at its window's first key
     reach = min(max_len, window) if window else max_len
@@ -914,8 +942,23 @@ def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
     _check(_fn("attn_capped", "mf_capped_attn")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(seq_of_tok),
         _ptr(temp), _ptr(out), _ptr(part), _is_bf16(q), n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale),
-        float(cap or 0.0), int(window or 0), int(chunk or 0), _ptr(far_a), _ptr(far_b), n_splits, split_len, _stream()),
-        "capped_attn")
+        float(cap or 0.0), int(window or 0), int(chunk or 0), _ptr(far_a), _ptr(far_b), keep_first, _ptr(bias), n_bias,
+        n_splits, split_len, _stream()), "capped_attn")
+
+
+def _kept_and_bias(what: str, keep_first, window, chunk, bias: Optional[torch.Tensor], n_heads: int):
+    """(keep_first, columns of the bias table) as the attention kernels take them, checked."""
+    keep_first = int(keep_first or 0)
+    if keep_first < 0 or (keep_first and chunk):
+        raise KernelError(f"{what}: keep_first {keep_first} with chunk {chunk}: kept first positions go with a window")
+    if not window:
+        keep_first = 0          # every earlier position is in sight anyway
+    if bias is None:
+        return keep_first, 0
+    _need(bias, what + ".bias", torch.float32)
+    if bias.dim() != 2 or bias.shape[0] != n_heads or bias.shape[1] < 1:
+        raise KernelError(f"{what}.bias: shape {tuple(bias.shape)}, expected [{n_heads}][distances]")
+    return keep_first, bias.shape[1]
 
 
 def _far_pair(what: str, far, n_heads: int):
@@ -938,7 +981,8 @@ def capped_mfma_takes(dtype, dim: int, v_dim: int) -> bool:
 
 def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor, ctx,
                         temp: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, v_dim: int,
-                        scale: float, cap: float, window: int, chunk: int = 0, far=None) -> None:
+                        scale: float, cap: float, window: int, chunk: int = 0, far=None, keep_first: int = 0,
+                        bias: Optional[torch.Tensor] = None) -> None:
     """`capped_attn` in bfloat16 on the matrix cores: blocks of 16 consecutive new tokens of a sequence
     (`ctx.query_tiles`) times the query heads of a kv head.  A decode step (one token a sequence) splits every
     token's keys over several waves (at least 128 keys a split) and merges the parts in their order."""
@@ -958,6 +1002,7 @@ def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Ten
     if ctx.max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"capped_attn_prefill: max_len {ctx.max_len} exceeds the page table")
     far_a, far_b = _far_pair("capped_attn_prefill", far, n_heads)
+    keep_first, n_bias = _kept_and_bias("capped_attn_prefill", keep_first, window, chunk, bias, n_heads)
     n_splits, split_len, part = 1, 0, None
     if ctx.all_decode:
         # every sequence is a tile of one token; nothing comes from the host (the step may be captured)
@@ -979,7 +1024,7 @@ def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Ten
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
         _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), tile_seq.numel(), _ptr(temp), _ptr(out), _ptr(part), n_splits,
         split_len, n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale), float(cap or 0.0), int(window or 0),
-        int(chunk or 0), _ptr(far_a), _ptr(far_b), _stream()),
+        int(chunk or 0), _ptr(far_a), _ptr(far_b), keep_first, _ptr(bias), n_bias, _stream()),
         "capped_attn_decode" if ctx.all_decode else "capped_attn_prefill")
 
 
@@ -989,13 +1034,18 @@ MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128     # what `moe_sparse` takes in o
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, dense: Optional[torch.Tensor], chosen: torch.Tensor,
-              weights: torch.Tensor, n_groups: int, keep: int, bias: Optional[torch.Tensor] = None) -> None:
+              weights: torch.Tensor, n_groups: int, keep: int, bias: Optional[torch.Tensor] = None,
+              score: str = "softmax", correction: Optional[torch.Tensor] = None, group_top: int = 1,
+              weight_scale: float = 1.0) -> None:
     """The router: logits = router x in 32-bit (`router` float32 `[experts][K]`, `x` `[tokens][K]` in the run
     type), softmax scores, the `keep` best of `n_groups` groups of neighbouring experts (a group's score is
     its best expert's), the `chosen.shape[1]` best experts of those groups, weighted by their scores over
     their sum.  `dense` `[tokens][experts]`, where given, gets the weights at the chosen experts and 0
     elsewhere; `chosen`, `weights` `[tokens][top]`.  `bias` float32 `[experts]` is added to the logits.  With one
-    group the weights are the softmax over the chosen logits alone."""
+    group the weights are the softmax over the chosen logits alone.  `score` "sigmoid": the scores are
+    sigmoid(logits).  `correction` float32 `[experts]` joins the scores where groups and experts are chosen, not in
+    the weights.  `group_top`: a group's score is the sum of its so many best (corrected) scores.  `weight_scale`
+    multiplies the weights."""
     n_tok, K = x.shape
     E = router.shape[0]
     top = chosen.shape[1]
@@ -1009,11 +1059,17 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, dense: Optional[torch.Tenso
         raise KernelError(f"moe_route: {E} experts in {n_groups} groups, {keep} kept, {top} chosen")
     if bias is not None:
         _need(bias, "moe_route.bias", torch.float32, (E,))
+    if correction is not None:
+        _need(correction, "moe_route.correction", torch.float32, (E,))
+    if score not in MOE_SCORES or group_top < 1:
+        raise KernelError(f"moe_route: scores {score!r} (one of {sorted(MOE_SCORES)}), group_top {group_top}")
     _check(_fn("moe", "mf_moe_route")(_ptr(x), _is_bf16(x), _ptr(router), _ptr(bias), K, _ptr(dense), _ptr(chosen), _ptr(weights),
-                                       n_tok, E, n_groups, keep, top, _stream()), "moe_route")
+                                       n_tok, E, n_groups, keep, top, MOE_SCORES[score], _ptr(correction), int(group_top),
+                                       float(weight_scale), _stream()), "moe_route")
 
 
 MOE_ACTS = {"clamped_swish": 0, "silu": 1}      # the experts' activations (MF_MOE_ACT_* in csrc/moe.hip)
+MOE_SCORES = {"softmax": 0, "sigmoid": 1}       # how a router turns logits into scores (MF_MOE_SCORE_*)
 
 
 def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: float, act: int = 0) -> None:
@@ -1109,17 +1165,29 @@ def mingru_scan(zug: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Ten
 def latent_prep(proj: torch.Tensor, off_dkv: int, off_gate: int, latent_weight: torch.Tensor, eps: float,
                 cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, seq_of_tok: torch.Tensor,
                 page_table: torch.Tensor, cache: torch.Tensor, q_plain: torch.Tensor, q_abs: torch.Tensor,
-                gate: torch.Tensor, n_heads: int, dim: int, rot_dim: int, rank: int, write_cache: bool = True) -> None:
+                gate: torch.Tensor, n_heads: int, dim: int, rot_dim: int, rank: int, write_cache: bool = True,
+                q_rows: Optional[torch.Tensor] = None) -> None:
     """From the 32-bit rows [q | dkv | gates] of one product: the normed latent and the rotated
     shared key part into the cache rows `[pages][64][rank + rot_dim]` at the tokens' positions, the
     plain query parts into `q_plain` `[tokens][heads][dim]`, the rotated query parts into the last
-    `rot_dim` columns of `q_abs` `[tokens][heads][rank + rot_dim]`, sigmoid of the gates into `gate`.
-    The tables have one column per rotated pair (2i, 2i+1); values behind the pairs pass unchanged."""
+    `rot_dim` columns of `q_abs` `[tokens][heads][rank + rot_dim]`, sigmoid of the gates into `gate`
+    (`[tokens][heads]`: one gate a head; `[tokens][heads][w]`: one for each of a head's w values).
+    The tables have one column per rotated pair (2i, 2i+1); values behind the pairs pass unchanged.
+    `q_rows`: the queries as 32-bit rows `[tokens][heads (dim + rot_dim)]` of their own, where they are not the
+    first columns of `proj`."""
     n_tok = positions.numel()
     ld = proj.shape[1]
     dk = rank + rot_dim
     _need(proj, "latent_prep.proj", torch.float32, (n_tok, ld))
-    if off_dkv < n_heads * (dim + rot_dim) or off_dkv + dk > ld or off_gate + n_heads > ld or off_gate < 0:
+    gate_w = 1 if gate.dim() == 2 else gate.shape[2]
+    if q_rows is None:
+        if off_dkv < n_heads * (dim + rot_dim):
+            raise KernelError(f"latent_prep: the queries do not fit in front of column {off_dkv}")
+        q_src = proj
+    else:
+        _need(q_rows, "latent_prep.q_rows", torch.float32, (n_tok, n_heads * (dim + rot_dim)))
+        q_src = q_rows
+    if off_dkv < 0 or off_dkv + dk > ld or off_gate + n_heads * gate_w > ld or off_gate < 0:
         raise KernelError(f"latent_prep: offsets {off_dkv}, {off_gate} do not fit rows of {ld}")
     _need(latent_weight, "latent_prep.latent_weight", torch.float32, (rank,))
     _need(cos, "latent_prep.cos", torch.float32)
@@ -1132,21 +1200,33 @@ def latent_prep(proj: torch.Tensor, off_dkv: int, off_gate: int, latent_weight: 
     _need(page_table, "latent_prep.page_table", torch.int32)
     _need(q_plain, "latent_prep.q_plain", _FLOATS, (n_tok, n_heads, dim))
     _need(q_abs, "latent_prep.q_abs", q_plain.dtype, (n_tok, n_heads, dk))
-    _need(gate, "latent_prep.gate", torch.float32, (n_tok, n_heads))
+    _need(gate, "latent_prep.gate", torch.float32, (n_tok, n_heads) if gate.dim() == 2 else (n_tok, n_heads, gate_w))
     _need(cache, "latent_prep.cache", q_plain.dtype)
     if cache.dim() < 2 or cache.shape[-1] != dk or cache.numel() % (PAGE * dk):
         raise KernelError(f"latent_prep: cache {tuple(cache.shape)} does not hold pages of {PAGE} rows of {dk}")
     _check(_fn("attn_latent", "mf_latent_prep")(
-        _ptr(proj), ld, off_dkv, off_gate, _ptr(latent_weight), float(eps), _ptr(cos), _ptr(sin), rd, _ptr(positions),
+        _ptr(proj), ld, off_dkv, off_gate, gate_w, _ptr(q_src), q_src.shape[1], _ptr(latent_weight), float(eps), _ptr(cos),
+        _ptr(sin), rd, _ptr(positions),
         _ptr(seq_of_tok), _ptr(page_table), page_table.shape[1], _ptr(cache), _ptr(q_plain), _ptr(q_abs), _ptr(gate),
         _is_bf16(q_plain), n_tok, n_heads, dim, rot_dim, rank, 1 if write_cache else 0, _stream()), "latent_prep")
+
+
+def _gate_width(what: str, gate: Optional[torch.Tensor], n_tok: int, heads: int, n_out: int) -> int:
+    """1 for a gate a head (`[tokens][heads]`) or none, `n_out` for a gate a value (`[tokens][heads][n_out]`)."""
+    if gate is None or gate.dim() == 2:
+        if gate is not None:
+            _need(gate, what + ".gate", torch.float32, (n_tok, heads))
+        return 1
+    _need(gate, what + ".gate", torch.float32, (n_tok, heads, n_out))
+    return n_out
 
 
 def headwise_linear(x: torch.Tensor, n_in: int, wt: torch.Tensor, out: torch.Tensor, n_out: int,
                     gate: Optional[torch.Tensor] = None) -> None:
     """out[t][h][:n_out] = (gate[t][h] *) wt[h]^T x[t][h][:n_in] for `wt` `[heads][n_in][n_out]` (each
     head's matrix stored input-major); x and out are `[tokens][heads][row]` with rows at least that
-    long, everything in the run type, sums in 32-bit."""
+    long, everything in the run type, sums in 32-bit.  A gate `[tokens][heads][n_out]` multiplies value by
+    value."""
     _need(x, "headwise_linear.x", _FLOATS)
     if x.dim() != 3 or out.dim() != 3:
         raise KernelError("headwise_linear: x and out are [tokens][heads][row]")
@@ -1157,10 +1237,9 @@ def headwise_linear(x: torch.Tensor, n_in: int, wt: torch.Tensor, out: torch.Ten
         raise KernelError(f"headwise_linear: x {tuple(x.shape)}, out {tuple(out.shape)}, matrix {tuple(wt.shape)}")
     if n_in * 32 > 64 * 1024:
         raise KernelError(f"headwise_linear: inputs of {n_in} values do not fit the kernel's staging")
-    if gate is not None:
-        _need(gate, "headwise_linear.gate", torch.float32, (n_tok, heads))
+    gate_w = _gate_width("headwise_linear", gate, n_tok, heads, n_out)
     _check(_fn("attn_latent", "mf_headwise_linear")(_ptr(x), in_stride, _ptr(wt), _ptr(out), out.shape[2], _ptr(gate),
-                                                     _is_bf16(x), n_tok, heads, n_in, n_out, _stream()),
+                                                     gate_w, _is_bf16(x), n_tok, heads, n_in, n_out, _stream()),
            "headwise_linear")
 
 
@@ -1183,10 +1262,9 @@ def headwise_linear_mfma(x: torch.Tensor, n_in: int, wo: torch.Tensor, out: torc
         raise KernelError(f"headwise_linear_mfma: x {tuple(x.shape)}, out {tuple(out.shape)}, matrix {tuple(wo.shape)}")
     if not headwise_mfma_takes(x.dtype, n_in, in_stride):
         raise KernelError(f"headwise_linear_mfma: inputs of {n_in} in rows of {in_stride} are not 16-byte pieces")
-    if gate is not None:
-        _need(gate, "headwise_linear_mfma.gate", torch.float32, (n_tok, heads))
+    gate_w = _gate_width("headwise_linear_mfma", gate, n_tok, heads, n_out)
     _check(_fn("attn_latent", "mf_headwise_mfma")(_ptr(x), in_stride, _ptr(wo), _ptr(out), out.shape[2], _ptr(gate),
-                                                   n_tok, heads, n_in, n_out, _stream()), "headwise_linear_mfma")
+                                                   gate_w, n_tok, heads, n_in, n_out, _stream()), "headwise_linear_mfma")
 
 
 def latent_split_plan(n_blocks: int, max_len: int, target_blocks: Optional[int] = None, most: int = 64) -> Tuple[int, int]:

@@ -155,6 +155,36 @@ class SandwichBlock(BranchNormBlock):
         return h
 
 
+@register_block("parallel_shared_norm")
+class SharedNormParallelBlock(Block):
+    """x + mixer(N(x)) + feed_forward(N(x)): one norm, whose output both branches read.  norms: "input"; a block
+    without a feed-forward is the mixer's branch alone.  The normed rows are made once, before the mixer adds
+    into the stream; where only some rows go on behind this block, the feed-forward gets the norm of those."""
+
+    needs_mixer = True
+    needs_feed_forward = False
+    norm_names = ("input",)
+
+    def first_norm(self):
+        return self.norms["input"]
+
+    def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
+        ctx.norm_next = ctx.norm_ahead = None
+        norm = self.norms["input"]
+        x = norm.forward(h)
+        x_ff = None
+        if self.feed_forward is not None:
+            x_ff = x if keep_rows is None else norm.forward(h, row_idx=keep_rows)
+        self.mixer.forward(x, h, ctx, entry, writes_cache)
+        if keep_rows is not None:
+            kept = torch.empty((keep_rows.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
+            ops.gather_rows(h, keep_rows, kept)
+            h = kept
+        if self.feed_forward is not None:
+            self.feed_forward.forward(x_ff, h, ctx)
+        return h
+
+
 @register_block("parallel")
 class ParallelBlock(Block):
     """x + mixer(N1(x)) + feed_forward(N2(x)): both branches read the same x, each through a norm of

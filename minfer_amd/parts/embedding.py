@@ -94,6 +94,22 @@ class LinearHead(Head):
         return self.linear(x, out_dtype=torch.float32)
 
 
+@register_head("capped_linear_head")
+class CappedLinearHead(LinearHead):
+    """The linear head with capped logits: z <- cap tanh(z / cap), in 32-bit.  params: those of `linear_head`, and cap."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.cap = float(spec.params["cap"])
+        if not self.cap > 0:
+            raise ValueError(f"capped_linear_head: cap {self.cap} must be positive")
+
+    def forward(self, x, ctx=None) -> torch.Tensor:
+        logits = super().forward(x, ctx)
+        ops.softcap(logits, self.cap)
+        return logits
+
+
 @register_embedding("token_position_embedding")
 class TokenPositionEmbedding(TokenEmbedding):
     """The table's row plus a learned row for the token's position (not scaled), added in 32-bit.

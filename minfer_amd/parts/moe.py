@@ -4,7 +4,9 @@ Router: z = Wr x in 32-bit, scores = softmax(z) over all experts; the experts fo
 groups of neighbours, a group's score is its best expert's, and only experts of the `keep` best groups
 can be among the `top` chosen; the chosen experts' scores over their sum are the weights.
 With one group (and so all of it kept) the weights are the softmax over the chosen logits alone.  A router may
-add a bias per expert to its logits.
+add a bias per expert to its logits.  A router may also score with sigmoid(z) instead of the softmax, choose
+groups and experts by score plus a correction per expert while weighing by the scores themselves, count a group
+by the sum of its `group_top` best (corrected) scores, and multiply the weights by a scale.
 Expert (no biases): g = min(Wg x, limit), u = clamp(Wu x, -limit, limit), y = g sigmoid(1.702 g) (u + 1),
 output Wd y; or, with `act` "silu", the plain gated form y = silu(Wg x) (Wu x).  The result is the weighted sum
 of the chosen experts' outputs.
@@ -36,8 +38,9 @@ SPARSE_UP_TO = ops.MOE_SPARSE_TOKENS
 class GroupedMoE(FeedForward):
     """params: hidden_size, intermediate_size (of one expert), n_experts, top, groups and keep (default 1: no
     groups), act ("clamped_swish", the default, with `limit`; or "silu"), router (tensor name), router_bias
-    (tensor name, or None), expert (format of an expert's tensor stem, e.g. "mlp.e{}"; its matrices are
-    stem + ".gate", ".up", ".down")."""
+    (tensor name, or None), score ("softmax", the default, or "sigmoid"), correction (tensor name, or None),
+    group_top (default 1), weight_scale (default 1.0), expert (format of an expert's tensor stem, e.g. "mlp.e{}";
+    its matrices are stem + ".gate", ".up", ".down")."""
 
     can_overwrite = True
 
@@ -54,16 +57,23 @@ class GroupedMoE(FeedForward):
         self.limit = float(p["limit"]) if act == "clamped_swish" else 0.0
         self.router_name, self.expert_name = p["router"], p["expert"]
         self.bias_name = p.get("router_bias")
+        self.correction_name = p.get("correction")
+        self.score, self.group_top = p.get("score", "softmax"), int(p.get("group_top", 1))
+        self.weight_scale = float(p.get("weight_scale", 1.0))
+        if self.score not in ops.MOE_SCORES or self.group_top < 1:
+            raise ValueError(f"grouped_moe: scores {self.score!r} (one of {sorted(ops.MOE_SCORES)}), group_top {self.group_top}")
         per = self.ne // max(1, self.groups)
         if self.ne % self.groups or not 1 <= self.keep <= self.groups or not 1 <= self.top <= min(64, self.keep * per) \
                 or self.ne > ops.MOE_MAX_EXPERTS:
             raise ValueError(f"grouped_moe: {self.ne} experts in {self.groups} groups, {self.keep} kept, {self.top} chosen")
-        self.router = self.router_bias = self.gate_up = self.down = None
+        self.router = self.router_bias = self.correction = self.gate_up = self.down = None
 
     def tensor_specs(self):
         s = {self.router_name: TensorSpec((self.ne, self.hidden))}
         if self.bias_name is not None:
             s[self.bias_name] = TensorSpec((self.ne,))
+        if self.correction_name is not None:
+            s[self.correction_name] = TensorSpec((self.ne,))
         for e in range(self.ne):
             stem = self.expert_name.format(e)
             s[stem + ".gate"] = TensorSpec((self.inter, self.hidden))
@@ -75,6 +85,8 @@ class GroupedMoE(FeedForward):
         self.router = get(self.router_name).to(torch.float32).contiguous()   # the router's product is 32-bit
         if self.bias_name is not None:
             self.router_bias = get(self.bias_name).to(torch.float32).contiguous()
+        if self.correction_name is not None:
+            self.correction = get(self.correction_name).to(torch.float32).contiguous()
         stems = [self.expert_name.format(e) for e in range(self.ne)]
         # [experts][gate | up][hidden] and [experts][hidden][inter]: an expert's matrices are contiguous slices
         self.gate_up = torch.stack([torch.cat([get(s + ".gate"), get(s + ".up")], dim=0) for s in stems]).contiguous()
@@ -88,7 +100,9 @@ class GroupedMoE(FeedForward):
         n, dev = x.shape[0], x.device
         chosen = torch.empty((n, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((n, self.top), dtype=torch.float32, device=dev)
-        ops.moe_route(x, self.router, None, chosen, weights, self.groups, self.keep, bias=self.router_bias)
+        ops.moe_route(x, self.router, None, chosen, weights, self.groups, self.keep, bias=self.router_bias,
+                      score=self.score, correction=self.correction, group_top=self.group_top,
+                      weight_scale=self.weight_scale)
         log = ctx._memo.get("route_log") if ctx is not None else None
         if log is not None:                  # a caller that wants to know: every routed layer's choices, in run order
             log.append(chosen)

@@ -48,6 +48,8 @@ def _register_builtin() -> None:
     register_architecture(lagedra.ARCHITECTURE, lagedra.LagedraConfig)
     from .config import nodutar
     register_architecture(nodutar.ARCHITECTURE, nodutar.NodutarConfig)
+    from .config import katarax
+    register_architecture(katarax.ARCHITECTURE, katarax.KataraxConfig)
 
 
 _register_builtin()

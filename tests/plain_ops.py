@@ -18,8 +18,10 @@ def embed(table, ids, out):
     out.copy_(table[ids.long()].to(torch.float32))
 
 
-def rmsnorm(x, weight, eps, out, row_idx=None):
+def rmsnorm(x, weight, eps, out, row_idx=None, cols=None):
     src = x if row_idx is None else x[row_idx.long()]
+    if cols is not None:
+        src = src[:, :cols]
     s = src.double()
     y = s * (1.0 / torch.sqrt((s * s).mean(dim=-1, keepdim=True) + eps))
     if weight is not None:
@@ -275,14 +277,14 @@ def mingru_scan(zug, cu_seqlens, slot_ids, state, out, chunks=None):
 
 # ------------------------------------------------------------------ latent attention
 def latent_prep(proj, off_dkv, off_gate, latent_weight, eps, cos, sin, positions, seq_of_tok, page_table, cache,
-                q_plain, q_abs, gate, n_heads, dim, rot_dim, rank, write_cache=True):
+                q_plain, q_abs, gate, n_heads, dim, rot_dim, rank, write_cache=True, q_rows=None):
     t = positions.numel()
     p = proj.double()
     c_t, s_t = cos[positions.long()].double(), sin[positions.long()].double()
-    q = p[:, :n_heads * (dim + rot_dim)].view(t, n_heads, dim + rot_dim)
+    q = (p if q_rows is None else q_rows.double())[:, :n_heads * (dim + rot_dim)].reshape(t, n_heads, dim + rot_dim)
     q_plain.copy_(q[:, :, :dim].to(q_plain.dtype))
     q_abs[:, :, rank:] = _rotate_pairs(q[:, :, dim:], c_t[:, None, :], s_t[:, None, :]).to(q_abs.dtype)
-    gate.copy_(torch.sigmoid(p[:, off_gate:off_gate + n_heads]).float())
+    gate.copy_(torch.sigmoid(p[:, off_gate:off_gate + gate[0].numel()]).float().view(gate.shape))
     if not write_cache:
         return
     c = p[:, off_dkv:off_dkv + rank]
@@ -300,7 +302,7 @@ def latent_prep(proj, off_dkv, off_gate, latent_weight, eps, cos, sin, positions
 def headwise_linear(x, n_in, wt, out, n_out, gate=None):
     y = torch.einsum("thi,hio->tho", x[:, :, :n_in].double(), wt.double())
     if gate is not None:
-        y = y * gate.double()[:, :, None]
+        y = y * (gate.double()[:, :, None] if gate.dim() == 2 else gate.double())
     out[:, :, :n_out] = y.to(out.dtype)
 
 
@@ -334,6 +336,10 @@ def embed_pos(table, pos_table, ids, positions, out):
 def gelu_tanh(x, out):
     z = x.double()
     out.copy_((0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))).to(out.dtype))
+
+
+def softcap(x, cap):
+    x.copy_((cap * torch.tanh(x.double() / cap)).float())
 
 
 def weighted_sum(buffers, weights, out, row_idx=None, n_indexed=0):
@@ -450,7 +456,7 @@ def qkv_conv_prep(qkv, conv_w, conv_state, cu_seqlens, seq_of_tok, slot_ids, pos
 
 
 def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out, n_heads, n_kv_heads, dim, v_dim,
-                scale, cap, window, max_len, chunk=0, far=None):
+                scale, cap, window, max_len, chunk=0, far=None, keep_first=0, bias=None):
     t_all = positions.numel()
     group = n_heads // n_kv_heads
     qq = q.double().view(t_all, n_heads, dim)
@@ -460,6 +466,8 @@ def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out,
         if chunk:
             lo = max(lo, p // chunk * chunk)
         pos = torch.arange(lo, p + 1)
+        if window and keep_first:
+            pos = torch.cat([torch.arange(0, min(keep_first, lo)), pos])
         pages = page_table[int(seq_of_tok[i])].long()[pos // PAGE]
         assert (pages >= 0).all(), "attention reads a page that was given back"
         for h in range(n_heads):
@@ -471,6 +479,8 @@ def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out,
                 s = cap * torch.tanh(s / cap)
             if far is not None:
                 s = s - float(far[0][h]) * torch.log1p(float(far[1][h]) * (p - pos).double())
+            if bias is not None:
+                s = s + bias[h].double()[torch.clamp(p - pos, max=bias.shape[1] - 1)]
             out[i, h * v_dim:(h + 1) * v_dim] = (torch.softmax(s, dim=0) @ vals).to(out.dtype)
 
 
@@ -479,9 +489,9 @@ def capped_mfma_takes(dtype, dim, v_dim):
 
 
 def capped_attn_prefill(q, kcache, vcache, page_table, ctx, temp, out, n_heads, n_kv_heads, dim, v_dim, scale, cap, window,
-                        chunk=0, far=None):
+                        chunk=0, far=None, keep_first=0, bias=None):
     capped_attn(q, kcache, vcache, page_table, ctx.positions, ctx.seq_of_tok, temp, out, n_heads, n_kv_heads, dim, v_dim,
-                scale, cap, window, ctx.max_len, chunk=chunk, far=far)
+                scale, cap, window, ctx.max_len, chunk=chunk, far=far, keep_first=keep_first, bias=bias)
 
 
 # ------------------------------------------------------------------ rows added into rows, the gated recurrence,
@@ -525,11 +535,14 @@ def head_rmsnorm(o, weight, eps, out, n_heads, scale=1.0):
 
 
 def qk_norm_prep(qkv, q_gain, k_gain, eps, normed, seq_of_tok, positions, rot_tables, value_tables, v_from_k, page_table,
-                 q_out, kcache, vcache, n_heads, n_kv_heads, dim, v_dim, write_cache=True):
+                 q_out, kcache, vcache, n_heads, n_kv_heads, dim, v_dim, write_cache=True, halves=False, q_only=False):
     t_all = positions.numel()
     y = qkv.double()
     nq, nk = n_heads * dim, n_kv_heads * dim
     q = y[:, :nq].view(t_all, n_heads, dim)
+    if q_only:           # no keys and values of its own: pad with zeros that nobody stores
+        y = torch.cat([y, torch.zeros(t_all, nk + n_kv_heads * v_dim, dtype=torch.float64)], dim=1)
+        write_cache = False
     k = y[:, nq:nq + nk].view(t_all, n_kv_heads, dim)
     v = k.clone() if v_from_k else y[:, nq + nk:].view(t_all, n_kv_heads, v_dim)
     if normed:
@@ -542,7 +555,8 @@ def qk_norm_prep(qkv, q_gain, k_gain, eps, normed, seq_of_tok, positions, rot_ta
     pos = positions.long()
     if rot_tables is not None:
         c, s = rot_tables[0][pos].double()[:, None, :], rot_tables[1][pos].double()[:, None, :]
-        q, k = _rotate_pairs(q, c, s), _rotate_pairs(k, c, s)
+        turn = _rotate_half_part if halves else _rotate_pairs
+        q, k = turn(q, c, s), turn(k, c, s)
     if value_tables is not None:
         v = _rotate_pairs(v, value_tables[0][pos].double()[:, None, :], value_tables[1][pos].double()[:, None, :])
     q_out.copy_(q.reshape(t_all, nq).to(q_out.dtype))
@@ -555,6 +569,13 @@ def qk_norm_prep(qkv, q_gain, k_gain, eps, normed, seq_of_tok, positions, rot_ta
         kcache[page, :, p % PAGE] = k[i].to(kcache.dtype)
         for g in range(n_kv_heads):
             _store_v(vcache, page, p % PAGE, g, v[i, g])
+
+
+def _rotate_half_part(v, c, s):
+    """Value i turns with value i + n, i < n = the tables' columns; the values from 2 n on pass."""
+    n = c.shape[-1]
+    a, b = v[..., :n], v[..., n:2 * n]
+    return torch.cat([a * c - b * s, b * c + a * s, v[..., 2 * n:]], dim=-1)
 
 
 def unrotate(rows, value_tables, positions, n_heads, scale=1.0):
@@ -574,7 +595,11 @@ MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128
 MOE_ACTS = {"clamped_swish": 0, "silu": 1}
 
 
-def moe_route(x, router, dense, chosen, weights, n_groups, keep, bias=None):
+MOE_SCORES = {"softmax": 0, "sigmoid": 1}
+
+
+def moe_route(x, router, dense, chosen, weights, n_groups, keep, bias=None, score="softmax", correction=None,
+              group_top=1, weight_scale=1.0):
     logits = x.double() @ router.double().t()
     if bias is not None:
         logits = logits + bias.double()
@@ -582,17 +607,18 @@ def moe_route(x, router, dense, chosen, weights, n_groups, keep, bias=None):
     n_tok, E = logits.shape
     top = chosen.shape[1]
     per = E // n_groups
-    s = torch.softmax(logits.float(), dim=-1)
+    s = torch.sigmoid(logits.float()) if score == "sigmoid" else torch.softmax(logits.float(), dim=-1)
+    choice = s if correction is None else s + correction.float()
     if dense is not None:
         dense.zero_()
     for t in range(n_tok):
-        gs = s[t].view(n_groups, per).max(dim=1).values
+        gs = torch.sort(choice[t].view(n_groups, per), dim=1, descending=True).values[:, :group_top].sum(dim=1)
         kept = torch.argsort(-gs, stable=True)[:keep]
-        masked = torch.full((E,), -1.0)
+        masked = torch.full((E,), float("-inf"))
         for g in kept.tolist():
-            masked[g * per:(g + 1) * per] = s[t, g * per:(g + 1) * per]
+            masked[g * per:(g + 1) * per] = choice[t, g * per:(g + 1) * per]
         pick = torch.argsort(-masked, stable=True)[:top]
-        w = s[t, pick] / (s[t, pick].sum() + 1e-20)
+        w = s[t, pick] / (s[t, pick].sum() + 1e-20) * weight_scale
         chosen[t] = pick.to(torch.int32)
         weights[t] = w
         if dense is not None:
@@ -728,7 +754,7 @@ NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", 
          "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma",
          "embed_pos", "gelu_tanh", "weighted_sum", "lightning_scan", "gated_rmsnorm", "rope_half_inplace",
          "qkv_conv_prep", "capped_attn", "capped_mfma_takes", "capped_attn_prefill", "moe_route", "moe_act", "moe_sparse", "moe_group", "moe_gather", "moe_combine",
-         "add_rows", "gr_chunks", "gated_scan", "head_rmsnorm", "qk_norm_prep", "unrotate"]
+         "add_rows", "gr_chunks", "gated_scan", "head_rmsnorm", "qk_norm_prep", "unrotate", "softcap"]
 
 
 def install(monkeypatch):
