@@ -138,7 +138,9 @@ def biased_window_attention(h, w, prefix: str, m):
     rel = w[prefix + "rel"]
     pos = np.arange(T)
     dist = pos[:, None] - pos[None, :]
-    seen = (dist >= 0) & ((dist < m["mask"]["size"]) | (pos[None, :] < m["mask"].get("keep_first", 0)))
+    seen = dist >= 0
+    if m.get("mask") is not None:          # no mask: every earlier position
+        seen = seen & ((dist < m["mask"]["size"]) | (pos[None, :] < m["mask"].get("keep_first", 0)))
     rows = np.array([[bucket(int(d), rel.shape[0], m["bias_max"]) if d >= 0 else 0 for d in r] for r in dist])
     bias = np.stack([rel[rows, hd] for hd in range(H)])
     return attend(q, k, v, seen, m["scale"], bias).reshape(T, H * V) @ w[prefix + "o"].T
@@ -159,7 +161,9 @@ def latent_attention(h, w, prefix: str, m, eps: float):
     q = np.concatenate([q[:, :, :D], q_rot], axis=-1)
     v = (c @ w[prefix + "uv"].T).reshape(T, H, V)
     dist = pos[:, None] - pos[None, :]
-    seen = (dist >= 0) & (dist < m["mask"]["size"])
+    seen = dist >= 0
+    if m.get("mask") is not None:
+        seen = seen & (dist < m["mask"]["size"])
     o = attend(q, k, v, seen, m["scale"]).reshape(T, H * V)
     return (o * sigmoid(h @ w[prefix + "g"].T)) @ w[prefix + "o"].T
 
