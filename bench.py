@@ -68,12 +68,12 @@ def parse():
                     help="cache size in tokens (default: batch x context, or what fits in free memory if less)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--only", choices=["decode", "prefill"], help="run one part (for profiles); prints no JSON line")
-    ap.add_argument("--design", choices=["tabezen", "lagedra", "nodutar"], default=None,
+    ap.add_argument("--design", choices=["tabezen", "lagedra", "nodutar", "katarax"], default=None,
                     help="instead of the default workload: prefill and decode of this design at a few layer sizes "
                          "beside its nearest relative of the same width, depth and feed-forward size (the Qwen2 "
                          "decoder; for nodutar, Lagedra), kernel by kernel")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes to run")
-    ap.add_argument("--design-model", default=None, choices=["tabezen", "lagedra", "nodutar", "qwen2"],
+    ap.add_argument("--design-model", default=None, choices=["tabezen", "lagedra", "nodutar", "katarax", "qwen2"],
                     help="with --design and --only: which of the two models runs the one part (for profiles; "
                          "default: the design itself)")
     return ap.parse_args()
@@ -285,6 +285,31 @@ def nodutar_config(width, layers, heads, ff, dim=128, vdim=128, chunk=1024, expe
                 layers=[dict(both if i % 2 == 0 else far, mlp=routed) for i in range(layers)])
 
 
+def katarax_config(width, layers, heads, ff, dim=128, vdim=128, window=1024, rank=512, rot_dim=64, experts=8, top=2, vocab=32768):
+    """Windowed attention with kept first positions and a bias by distance, windowed latent attention, causal
+    attention with unit queries and keys, and a layer that reads that one's keys and values, in turn; every layer
+    with routed experts of ff / top values, `top` of them a token; head sizes, kv heads and the window (Nodutar's
+    chunk) as in `nodutar_config`, the latent as in `tabezen_config`."""
+    kv = max(1, heads // 4)
+    biased = dict(type="attention", mixer=dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=dim ** -0.5, bias_max=2048,
+                                               bias_rows=32, mask=dict(size=window, keep_first=4)))
+    lat = dict(type="latent_attention", mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=rank,
+                                                   q_rank=3 * width // 8, scale=(dim + rot_dim) ** -0.5,
+                                                   rot=dict(base=10000.0, dims=rot_dim), mask=dict(size=window)))
+    own = dict(type="attention_2", mixer=dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=dim ** -0.5 * 8.0,
+                                              rot=dict(base=10000.0, dims=dim)))
+    routed = dict(kind="moe", expert=dict(ff=ff // top, limit=7.0),
+                  router=dict(experts=experts, top=top, scale=2.5, groups=dict(count=4, keep=2)))
+    made = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 3:
+            made.append(dict(type="attention_2", mixer=dict(own["mixer"], kv_from=i - 1), mlp=routed))
+        else:
+            made.append(dict((biased, lat, own)[kind], mlp=routed))
+    return dict(architecture="Katarax", vocab=vocab, width=width, norm=dict(eps=1e-6), logit_softcap=30.0, layers=made)
+
+
 def qwen2_like(width, layers, heads, ff, vocab=32768):
     """The Qwen2 decoder of the same width, depth, head count and feed-forward size (head size 128)."""
     return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
@@ -298,8 +323,10 @@ DESIGN_SIZES = {
 }
 
 
-DESIGN_CONFIGS = {"tabezen": tabezen_config, "lagedra": lagedra_config, "nodutar": nodutar_config, "qwen2": qwen2_like}
-NEAREST = {"tabezen": "qwen2", "lagedra": "qwen2", "nodutar": "lagedra"}      # the model a design is measured beside
+DESIGN_CONFIGS = {"tabezen": tabezen_config, "lagedra": lagedra_config, "nodutar": nodutar_config, "katarax": katarax_config,
+                  "qwen2": qwen2_like}
+# the model a design is measured beside
+NEAREST = {"tabezen": "qwen2", "lagedra": "qwen2", "nodutar": "lagedra", "katarax": "nodutar"}
 
 
 def traced_step(eng, slots, toks, want):

@@ -24,8 +24,9 @@
 // [H (DN + DR)] are rows of `ldq` floats of `q_rows` (the same buffer where one product made them all, or the
 // result of a product of their own where the queries pass a latent first).  gate_w: 1 where a head has one gate,
 // the width of a head's values where every value has its own.  Two blocks per token: one for the cached row,
-// one for the queries and gates.
-template <typename OT>
+// one for the queries and gates.  WIDE: the queries are rows of their own or a head has more than one gate; without
+// it the kernel is the one-product, one-gate-a-head form, instruction for instruction.
+template <typename OT, bool WIDE>
 __global__ __launch_bounds__(256) void latent_prep_kernel(
     const float* __restrict__ proj, int ld, int off_dkv, int off_gate, int gate_w, const float* __restrict__ q_rows,
     int ldq, const float* __restrict__ cw, float eps,
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
   const int DQ = DN + DR;
   for (int i = threadIdx.x; i < H * DQ; i += 256) {
     const int h = i / DQ, e = i % DQ;
-    const float* qh = q_rows + (size_t)t * ldq + (size_t)h * DQ;
+    const float* qh = WIDE ? q_rows + (size_t)t * ldq + (size_t)h * DQ : row + (size_t)h * DQ;
     if (e < DN) {
       q_plain[((size_t)t * H + h) * DN + e] = from_f32<OT>(qh[e]);
     } else {
@@ -85,9 +86,13 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
       q_abs[((size_t)t * H + h) * DK + R + j] = from_f32<OT>(v);
     }
   }
-  if (gate)
-    for (int i = threadIdx.x; i < H * gate_w; i += 256)
-      gate[(size_t)t * H * gate_w + i] = 1.0f / (1.0f + expf(-row[off_gate + i]));
+  if (WIDE) {
+    if (gate)
+      for (int i = threadIdx.x; i < H * gate_w; i += 256)
+        gate[(size_t)t * H * gate_w + i] = 1.0f / (1.0f + expf(-row[off_gate + i]));
+  } else {
+    for (int h = threadIdx.x; h < H; h += 256) gate[(size_t)t * H + h] = 1.0f / (1.0f + expf(-row[off_gate + h]));
+  }
 }
 
 MF_API int mf_latent_prep(const float* proj, int ld, int off_dkv, int off_gate, int gate_w, const float* q_rows,
@@ -98,17 +103,20 @@ MF_API int mf_latent_prep(const float* proj, int ld, int off_dkv, int off_gate, 
                           hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (rd < 0 || rd > DR || (rd & 1) || H < 1 || DN < 1 || R < 1 || gate_w < 1 || !q_rows) return (int)hipErrorInvalidValue;
-  if (is_bf16)
-    latent_prep_kernel<bf16><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, gate_w, q_rows, ldq, cw, eps, cs, sn, rd,
-                                                         positions,
-                                                         seq_of_tok, page_table, pt_stride, (bf16*)cache,
-                                                         (bf16*)q_plain, (bf16*)q_abs, gate, H, DN, DR, R, write_cache);
-  else
-    latent_prep_kernel<float><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, gate_w, q_rows, ldq, cw, eps, cs, sn, rd,
-                                                         positions,
-                                                          seq_of_tok, page_table, pt_stride, (float*)cache,
-                                                          (float*)q_plain, (float*)q_abs, gate, H, DN, DR, R,
-                                                          write_cache);
+  const bool wide = gate_w != 1 || q_rows != proj || ldq != ld || !gate;
+#define MF_PREP(OT, WIDE)                                                                                              \
+  latent_prep_kernel<OT, WIDE><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, gate_w, q_rows, ldq, cw, eps, \
+                                                                   cs, sn, rd, positions, seq_of_tok, page_table,      \
+                                                                   pt_stride, (OT*)cache, (OT*)q_plain, (OT*)q_abs,   \
+                                                                   gate, H, DN, DR, R, write_cache)
+  if (is_bf16) {
+    if (wide) MF_PREP(bf16, true);
+    else MF_PREP(bf16, false);
+  } else {
+    if (wide) MF_PREP(float, true);
+    else MF_PREP(float, false);
+  }
+#undef MF_PREP
   return mf_launch_status();
 }
 
@@ -118,7 +126,7 @@ MF_API int mf_latent_prep(const float* proj, int ld, int off_dkv, int off_gate, 
 // `in` and `out` are H slices of `in_stride` / `out_stride` values.  A block takes TT tokens of one
 // head; sums in 32-bit in the order of i.
 #define MF_HW_TT 8
-template <typename T>
+template <typename T, bool GV>          // GV: a gate for every value of a head (gate_w = NO) instead of one a head
 __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restrict__ in, int in_stride,
                                                               const T* __restrict__ wt, T* __restrict__ out,
                                                               int out_stride, const float* __restrict__ gate,
@@ -145,7 +153,7 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restric
 #pragma unroll
     for (int tt = 0; tt < MF_HW_TT; ++tt)
       if (tt < nt) {
-        const float g = gate ? gate[((size_t)(t0 + tt) * H + h) * gate_w + (gate_w > 1 ? o : 0)] : 1.0f;
+        const float g = gate ? (GV ? gate[((size_t)(t0 + tt) * H + h) * gate_w + o] : gate[(size_t)(t0 + tt) * H + h]) : 1.0f;
         out[((size_t)(t0 + tt) * H + h) * out_stride + o] = from_f32<T>(acc[tt] * g);
       }
   }
@@ -158,12 +166,18 @@ MF_API int mf_headwise_linear(const void* in, int in_stride, const void* wt, voi
   const size_t lds = (size_t)MF_HW_TT * NI * sizeof(float);
   if (H < 1 || NI < 1 || NO < 1 || lds > 64 * 1024 || (gate && gate_w != 1 && gate_w != NO)) return (int)hipErrorInvalidValue;
   dim3 grid((n_tok + MF_HW_TT - 1) / MF_HW_TT, H, (NO + 255) / 256);
-  if (is_bf16)
-    headwise_linear_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)in, in_stride, (const bf16*)wt, (bf16*)out,
-                                                              out_stride, gate, gate_w, n_tok, H, NI, NO);
-  else
-    headwise_linear_kernel<float><<<grid, 256, lds, stream>>>((const float*)in, in_stride, (const float*)wt,
-                                                               (float*)out, out_stride, gate, gate_w, n_tok, H, NI, NO);
+  const bool gv = gate && gate_w > 1;
+#define MF_HW(T, GV)                                                                                                  \
+  headwise_linear_kernel<T, GV><<<grid, 256, lds, stream>>>((const T*)in, in_stride, (const T*)wt, (T*)out, out_stride, gate, \
+                                                            gate_w, n_tok, H, NI, NO)
+  if (is_bf16) {
+    if (gv) MF_HW(bf16, true);
+    else MF_HW(bf16, false);
+  } else {
+    if (gv) MF_HW(float, true);
+    else MF_HW(float, false);
+  }
+#undef MF_HW
   return mf_launch_status();
 }
 
@@ -176,7 +190,7 @@ MF_API int mf_headwise_linear(const void* in, int in_stride, const void* wt, voi
 // head's rows of W where the step has tokens enough, and spread over the outputs where not.
 typedef unsigned int hw_u32x4 __attribute__((ext_vector_type(4)));
 
-template <int MT>
+template <int MT, bool GV>
 __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restrict__ in, int in_stride,
                                                             const bf16* __restrict__ wo, bf16* __restrict__ out,
                                                             int out_stride, const float* __restrict__ gate, int gate_w,
@@ -215,8 +229,8 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
     }
   }
   if (!tok_ok) return;
-  const float* grow = gate ? gate + ((size_t)t * H + h) * gate_w : nullptr;
-  const float g = (gate && gate_w == 1) ? grow[0] : 1.0f;
+  const float* grow = (GV && gate) ? gate + ((size_t)t * H + h) * gate_w : nullptr;
+  const float g = (!GV && gate) ? gate[(size_t)t * H + h] : 1.0f;
   bf16* orow = out + ((size_t)t * H + h) * out_stride;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -224,12 +238,12 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
     if (o0 + 3 < NO && (out_stride & 3) == 0) {
       bf16x4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[mt][i] * (gate_w > 1 ? grow[o0 + i] : g));
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[mt][i] * (GV ? grow[o0 + i] : g));
       *reinterpret_cast<bf16x4*>(orow + o0) = v;
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[mt][i] * (gate_w > 1 ? grow[o0 + i] : g));
+        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[mt][i] * (GV ? grow[o0 + i] : g));
     }
   }
 }
@@ -240,6 +254,7 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
 // (rows 16 bytes apart in the banks).  The matrix is read from memory once per 128 tokens
 // instead of once per 16.
 #define MF_HW_KS_MAX 16
+template <bool GV>
 __global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restrict__ in, int in_stride,
                                                            const bf16* __restrict__ wo, bf16* __restrict__ out,
                                                            int out_stride, const float* __restrict__ gate, int gate_w,
@@ -271,8 +286,8 @@ __global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restric
     if (ks < nks && tok_ok && i < NI) xb[ks] = *reinterpret_cast<const hw_u32x4*>(xrow + i);
   }
   if (blockIdx.x * 128 + wv * 16 >= n_tok) return;      // (after the barrier; uniform over the wave)
-  const float* grow = (gate && tok_ok) ? gate + ((size_t)t * H + h) * gate_w : nullptr;
-  const float g = (grow && gate_w == 1) ? grow[0] : 1.0f;
+  const float* grow = (GV && gate && tok_ok) ? gate + ((size_t)t * H + h) * gate_w : nullptr;
+  const float g = (!GV && gate && tok_ok) ? gate[(size_t)t * H + h] : 1.0f;
   bf16* orow = out + ((size_t)(tok_ok ? t : 0) * H + h) * out_stride;
   for (int mt = 0; mt < NO16 / 16; ++mt) {
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -291,12 +306,12 @@ __global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restric
     if (o0 + 3 < NO && (out_stride & 3) == 0) {
       bf16x4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[i] * (gate_w > 1 ? grow[o0 + i] : g));
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[i] * (GV ? grow[o0 + i] : g));
       *reinterpret_cast<bf16x4*>(orow + o0) = v;
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[i] * (gate_w > 1 ? grow[o0 + i] : g));
+        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[i] * (GV ? grow[o0 + i] : g));
     }
   }
 }
@@ -309,29 +324,41 @@ MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void*
     return (int)hipErrorInvalidValue;
   const int n_ttiles = (n_tok + 15) / 16;
   const size_t lds = (size_t)((NO + 15) / 16 * 16) * (NI + 8) * 2;
+  const bool gv = gate && gate_w > 1;
   if (n_tok >= 256 && NI <= 32 * MF_HW_KS_MAX && lds <= 150 * 1024) {
     static bool raised = false;
     if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(headwise_lds_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-      if (e != hipSuccess) return (int)e;
+      for (const void* fn : {reinterpret_cast<const void*>(headwise_lds_kernel<false>),
+                             reinterpret_cast<const void*>(headwise_lds_kernel<true>)}) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        if (e != hipSuccess) return (int)e;
+      }
       raised = true;
     }
-    headwise_lds_kernel<<<dim3((n_tok + 127) / 128, H), 512, lds, stream>>>(
-        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO);
+    const dim3 grid((n_tok + 127) / 128, H);
+    if (gv)
+      headwise_lds_kernel<true><<<grid, 512, lds, stream>>>((const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride,
+                                                           gate, gate_w, n_tok, H, NI, NO);
+    else
+      headwise_lds_kernel<false><<<grid, 512, lds, stream>>>((const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride,
+                                                            gate, gate_w, n_tok, H, NI, NO);
     return mf_launch_status();
   }
+#define MF_HWM(MT, GV)                                                                                                     \
+  headwise_mfma_kernel<MT, GV><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(                                           \
+      (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO, n_ttiles, n_otiles)
   if (n_tok <= 16) {
     const int n_otiles = (NO + 15) / 16;
     const long long tasks = (long long)H * n_otiles * n_ttiles;
-    headwise_mfma_kernel<1><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(
-        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO, n_ttiles, n_otiles);
+    if (gv) MF_HWM(1, true);
+    else MF_HWM(1, false);
   } else {
     const int n_otiles = (NO + 63) / 64;
     const long long tasks = (long long)H * n_otiles * n_ttiles;
-    headwise_mfma_kernel<4><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(
-        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, gate_w, n_tok, H, NI, NO, n_ttiles, n_otiles);
+    if (gv) MF_HWM(4, true);
+    else MF_HWM(4, false);
   }
+#undef MF_HWM
   return mf_launch_status();
 }
 
