@@ -58,18 +58,19 @@ class LatentAttention(Mixer):
 
     def tensor_specs(self):
         n, H = self.names, self.nh
-        s = {n["dkv"]: TensorSpec((self.dk, self.hidden)),
-             n["dkv_norm"]: TensorSpec((self.rank,), init="ones"),
-             n["uk"]: TensorSpec((H * self.dn, self.rank)),
-             n["uv"]: TensorSpec((H * self.dv, self.rank)),
-             n["gate"]: TensorSpec((H * self.gate_w, self.hidden)),
-             n["o"]: TensorSpec((self.hidden, H * self.dv))}
+        s = {}
         if self.q_rank is None:
             s[n["q"]] = TensorSpec((H * (self.dn + self.dr), self.hidden))
         else:
             s[n["dq"]] = TensorSpec((self.q_rank, self.hidden))
             s[n["dq_norm"]] = TensorSpec((self.q_rank,), init="ones")
             s[n["q"]] = TensorSpec((H * (self.dn + self.dr), self.q_rank))
+        s.update({n["dkv"]: TensorSpec((self.dk, self.hidden)),
+                  n["dkv_norm"]: TensorSpec((self.rank,), init="ones"),
+                  n["uk"]: TensorSpec((H * self.dn, self.rank)),
+                  n["uv"]: TensorSpec((H * self.dv, self.rank)),
+                  n["gate"]: TensorSpec((H * self.gate_w, self.hidden)),
+                  n["o"]: TensorSpec((self.hidden, H * self.dv))})
         return s
 
     def load(self, get):

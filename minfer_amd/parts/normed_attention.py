@@ -112,11 +112,12 @@ class NormedAttention(Mixer):
 
     def tensor_specs(self):
         n = self.names
-        s = {n["q"]: TensorSpec((self.nh * self.dim, self.hidden)), n["o"]: TensorSpec((self.hidden, self.nh * self.vdim))}
+        s = {n["q"]: TensorSpec((self.nh * self.dim, self.hidden))}
         if not self.shared_kv:
             s[n["k"]] = TensorSpec((self.nk * self.dim, self.hidden))
-            if not self.v_from_k:
-                s[n["v"]] = TensorSpec((self.nk * self.vdim, self.hidden))
+        s[n["o"]] = TensorSpec((self.hidden, self.nh * self.vdim))
+        if not self.shared_kv and not self.v_from_k:
+            s[n["v"]] = TensorSpec((self.nk * self.vdim, self.hidden))
         if self.bias_spec is not None:
             s[self.bias_spec["table"]] = TensorSpec((int(self.bias_spec["rows"]), self.nh))
         if self.gains:
