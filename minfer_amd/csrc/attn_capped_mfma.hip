@@ -38,6 +38,31 @@ constexpr int NVT = V / 16;            // output tiles
 static_assert(D % 16 == 0 && V % 16 == 0 && D <= 256 && V <= 256, "sizes the kernel takes");
 
 typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));      // four floats from any float's address
+
+// out[j] = row[clamp(d0 - j, 0, n - 1)], j < 4: the numbers a head's row holds for four neighbouring keys' distances,
+// fetched as one run of four floats (the run is moved inside the row at its ends, and every value picked by its
+// place in the run)
+__device__ __forceinline__ void bias_run(const float* __restrict__ row, int n, int d0, float (&out)[4]) {
+  if (__all(d0 >= 3 && d0 < n)) {        // every lane's run lies inside its row: the values as they come, last first
+    const float4u v = *(const float4u*)(row + d0 - 3);
+    out[0] = v[3];
+    out[1] = v[2];
+    out[2] = v[1];
+    out[3] = v[0];
+  } else if (n >= 4) {
+    const int start = min(max(d0 - 3, 0), n - 4);
+    const float4u v = *(const float4u*)(row + start);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int o = min(max(d0 - j, 0), n - 1) - start;
+      out[j] = o == 0 ? v[0] : (o == 1 ? v[1] : (o == 2 ? v[2] : v[3]));
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = row[min(max(d0 - j, 0), n - 1)];
+  }
+}
 
 __device__ __forceinline__ float fast_tanh(float y) {
   // 1 - 2 / (e^(2y) + 1), exact at both ends
@@ -155,13 +180,11 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     // which of this lane's 8 keys its token sees: slot j < 4: key kb + 4 g + j, else kb + 16 + 4 g + j - 4
     bool seen[8];
     float dist[8];
-    int far_row[8];      // the distance's place in a head's row of the bias table
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int key = kb + (j < 4 ? 4 * g + j : 16 + 4 * g + j - 4);
       seen[j] = row_ok && key <= p_mine && (window <= 0 || p_mine - key < window || key < keep_first) && key >= chunk_lo;
       dist[j] = (float)max(0, p_mine - key);
-      far_row[j] = min(max(0, p_mine - key), n_bias - 1);
     }
     bf16x8 pf[RB];
 #pragma unroll
@@ -174,12 +197,18 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
       }
       float x[8];
       float mx = -INFINITY;
+      float add_lo[4] = {0.f, 0.f, 0.f, 0.f}, add_hi[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {        // this lane's keys are two runs of four neighbours, 16 keys apart
+        const float* brow = bias + (size_t)(h0 + r) * n_bias;
+        bias_run(brow, n_bias, p_mine - (kb + 4 * g), add_lo);
+        bias_run(brow, n_bias, p_mine - (kb + 16 + 4 * g), add_hi);
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         float y = (j < 4 ? s0[j] : s1[j - 4]) * sc[r];
         if (cap > 0.f) y = cap * fast_tanh(y * inv_cap);
         if (far_a) y -= fa[r] * __logf(1.0f + fb[r] * dist[j]);
-        if (bias) y += bias[(size_t)(h0 + r) * n_bias + far_row[j]];
+        if (bias) y += j < 4 ? add_lo[j] : add_hi[j - 4];
         x[j] = seen[j] ? y : -INFINITY;
         mx = fmaxf(mx, x[j]);
       }
