@@ -311,6 +311,24 @@ def test_replays_agree_with_plain(folders, plains, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_in_which_nothing_or_little_is_wanted(folders, plains, dtype):
+    """A prompt step that asks for no logits at all, then single tokens of which one sequence's are wanted."""
+    eng = engine_for(folders["A"], dtype)
+    toks = random_tokens(300, 100, 5)
+    a, b = eng.new_sequence(), eng.new_sequence()
+    assert tuple(eng.step([a, b], [toks[:90], toks[:50]], [[], []]).shape) == (0, 300)
+    got_a = eng.step([a, b], [toks[90:91], toks[50:51]], [[0], []]).cpu().numpy()
+    got_b = eng.step([a, b], [toks[91:92], toks[51:52]], [[], [0]]).cpu().numpy()
+    assert got_a.shape == (1, 300) and got_b.shape == (1, 300)
+    for got, n in ((got_a, 91), (got_b, 52)):
+        want = plains["A"].forward(toks[:n])[-1]
+        tol = F32_ABS * max(1.0, want.std()) if dtype == "float32" else SHARP * BF16_MAX * want.std()
+        assert np.abs(got[0] - want).max() <= tol
+    eng.end_sequence(a)
+    eng.end_sequence(b)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_batch_of_more_sequences_than_one_launch_of_the_experts_takes(folders, plains, dtype):
     """Twenty sequences that start and decode together: the routed layers' few-token form runs in slices."""
     reqs = requests_for(KT["A"]["vocab"], tuple(3 + (7 * i) % 11 for i in range(20)), seed=12)
