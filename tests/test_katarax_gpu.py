@@ -93,7 +93,7 @@ _WANT = {}
 @pytest.mark.parametrize("H, G, D, V, window, keep, n_bias", [
     (6, 3, 32, 48, 17, 3, 9), (8, 2, 96, 48, 0, 0, 40), (4, 4, 16, 16, 64, 64, 0), (8, 2, 128, 64, 70, 5, 300),
     (7, 7, 48, 16, 1, 33, 2), (6, 2, 48, 48, 100, 1, 1), (6, 2, 128, 128, 65, 70, 0), (2, 1, 64, 128, 33, 32, 500),
-    (9, 1, 10, 6, 5, 2, 7), (3, 3, 20, 12, 40, 130, 11)])
+    (9, 1, 10, 6, 5, 2, 7), (3, 3, 20, 12, 40, 130, 11), (4, 2, 256, 256, 40, 3, 50), (4, 4, 192, 80, 100, 0, 9)])
 @pytest.mark.parametrize("new", [(1, 130, 3, 1, 40), (1, 64, 64, 300, 65), (1, 1, 1, 1, 1)])
 def test_window_kept_first_positions_and_bias_in_both_attention_kernels(form, dtype, H, G, D, V, window, keep, n_bias, new):
     """Prompts, portions on held tokens and single tokens in one launch, over shuffled pages of a poisoned pool."""
